@@ -1,0 +1,167 @@
+/*
+ * kraken_amd.h — C ABI of libkraken_amd.so
+ *
+ * The local (one-rank) arithmetic of Kraken's fused communication+compute
+ * kernels, written for AMD MI355X (gfx950).  The W peer symmetric-memory
+ * buffers of the reference are replaced by W slices of one device tensor
+ * ("stack"): slice r starts at  stack + r * slice_stride  elements.
+ *
+ * Conventions for every entry point
+ *   - all data pointers are DEVICE pointers; bf16 = 2-byte bfloat16;
+ *   - `stream` is a hipStream_t (NULL = the default stream); a call enqueues
+ *     its kernel(s) on that stream and returns without synchronising;
+ *   - the library keeps no state between calls and is re-entrant;
+ *   - return value: 0 on success; a negative KR_ERR_* code when the arguments
+ *     are rejected on the host BEFORE anything is launched (so argument
+ *     validation can be exercised on a machine without a GPU); a positive
+ *     value is a hipError_t reported by the launch.
+ *   - accumulation is fp32 in ascending slice order r = 0..W-1, and results
+ *     are rounded to bf16 once (round-to-nearest-even) at the store.
+ *
+ * The reference has no FFI layer: each function below names the Triton kernel
+ * and host wrapper of the reference whose arithmetic it replaces.
+ */
+#ifndef KRAKEN_AMD_H
+#define KRAKEN_AMD_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* argument errors (returned before any launch) */
+#define KR_OK                 0
+#define KR_ERR_NULL_POINTER  -1  /* a required pointer is NULL                      */
+#define KR_ERR_ALIGNMENT     -2  /* pointer or stride not 16-byte aligned           */
+#define KR_ERR_NUMEL_MOD8    -3  /* element count not a multiple of 8 (128 bit)     */
+#define KR_ERR_BAD_DIM       -4  /* negative/zero/inconsistent dimension            */
+#define KR_ERR_WORLD_SIZE    -5  /* W outside 1..KR_MAX_WORLD                       */
+#define KR_ERR_BIAS_SHAPE    -6  /* bias_numel is neither numel nor D               */
+#define KR_ERR_ROW_TOO_LONG  -7  /* D above KR_MAX_ROW for the row-resident kernels */
+#define KR_ERR_BAND          -8  /* row band outside [0, M) or M % W != 0           */
+#define KR_ERR_LAYOUT        -9  /* operand strides not supported                   */
+#define KR_ERR_STRIPE       -10  /* stripe block not a multiple of 8 / bad rank     */
+
+#define KR_MAX_WORLD 16
+#define KR_MAX_ROW   65536
+
+/* Library/ABI version: major*10000 + minor*100 + patch. */
+int kr_version(void);
+
+/* Human-readable text for a return code of this library (never NULL). */
+const char* kr_strerror(int code);
+
+/*
+ * W-way elementwise reduce with optional bias.
+ *   out[i] = bf16( [bias] + sum_{r=0..W-1} fp32(stack[r*slice_stride + i]) ),  0 <= i < numel
+ * bias == NULL: plain sum.  Otherwise bias_numel is either numel (bias has
+ * the shape of the input, as the reference passes it) or D (a vector
+ * broadcast over rows of length D, numel % D == 0).
+ * bias_first != 0: acc starts at bias, slices added after (one-shot order);
+ * bias_first == 0: slices summed from 0.0f, bias added last (two-shot order).
+ * Requirements: numel % 8 == 0, D % 8 == 0, slice_stride % 8 == 0, all
+ * pointers 16-byte aligned, 1 <= W <= KR_MAX_WORLD.  numel == 0 is a no-op.
+ *
+ * Replaces the reduce loops of
+ *   kraken/comm/one_shot_all_reduce.py:36-48          (one_shot_all_reduce_kernel)
+ *   kraken/comm/two_shot_all_reduce.py:51-62          (own share of two_shot_all_reduce_kernel)
+ *   kraken/fused/one_shot_all_reduce_bias.py:76-94    (one_shot_all_reduce_bias_kernel)
+ *   kraken/fused/two_shot_all_reduce_bias.py:66-83    (two_shot_all_reduce_bias_kernel)
+ * A two-shot share is this call with `stack`, `bias` and `numel` restricted
+ * to the rank's contiguous chunk.
+ */
+int kr_reduce_bf16(const void* stack, int W, int64_t slice_stride, int64_t numel,
+                   const void* bias, int64_t bias_numel, int64_t D, int bias_first,
+                   void* out, void* stream);
+
+/*
+ * Two-shot share with the reference's interleaved ownership: the flat input is
+ * cut into stripes of stripe_block*W elements and rank `rank` owns elements
+ * [rank*stripe_block, (rank+1)*stripe_block) of every stripe
+ * (kraken/comm/two_shot_all_reduce.py:51-54, kraken/fused/two_shot_all_reduce_bias.py:66-69).
+ * The owned elements (those below numel) are reduced (bias, if given, has
+ * numel elements and is added last) and written COMPACTLY to out in ascending
+ * order; *the caller sizes out* with kr_striped_share_numel().
+ * Requirements as kr_reduce_bf16 plus stripe_block % 8 == 0, 0 <= rank < W.
+ */
+int kr_reduce_striped_bf16(const void* stack, int W, int64_t slice_stride, int64_t numel,
+                           const void* bias, int64_t stripe_block, int rank,
+                           void* out, void* stream);
+
+/* Number of elements rank `rank` owns under the striped ownership above
+ * (negative KR_ERR_* on bad arguments). */
+int64_t kr_striped_share_numel(int64_t numel, int W, int64_t stripe_block, int rank);
+
+/*
+ * W-way reduce + bias + RMSNorm, one pass over the input.  For each of `rows`
+ * rows of length D:
+ *   s[c] = [bias] + sum_{r=0..W-1} fp32(stack[r*slice_stride + row*D + c])     (fp32, bias first)
+ *   y[row*D + c] = bf16( s[c] * rsqrt(mean_c(s^2) + eps) * fp32(w[c]) )
+ * bias: NULL, or [rows*D] (bias_is_vector == 0), or [D] (bias_is_vector != 0).
+ * w: [D] bf16.  Requirements: D % 8 == 0, D <= KR_MAX_ROW, slice_stride % 8 == 0.
+ *
+ * Replaces kraken/fused/one_shot_all_reduce_bias_rms_norm.py:73-91
+ * and      kraken/fused/two_shot_all_reduce_bias_rms_norm.py:87-94,110-121
+ * (the row is kept in fp32 registers between the reduce and the norm; the
+ * reference's two-shot variant rounds it to bf16 in between).
+ */
+int kr_reduce_rmsnorm_bf16(const void* stack, int W, int64_t slice_stride, int64_t rows, int64_t D,
+                           const void* bias, int bias_is_vector, const void* w, float eps,
+                           void* y, void* stream);
+
+/*
+ * Stand-alone RMSNorm: y = bf16( x * rsqrt(mean(x^2) + eps) * w ), row-wise.
+ * Replaces kraken/fused/rms_norm.py:34-43 (_rms_norm_kernel).
+ */
+int kr_rmsnorm_bf16(const void* x, const void* w, float eps, int64_t rows, int64_t D,
+                    void* y, void* stream);
+
+/*
+ * bf16 GEMM (fp32 accumulate on the matrix cores) with a fused reduce(+bias)
+ * epilogue:
+ *   C = A[M,K] @ B[K,N]
+ *   for rows m in [band_row0, band_row0 + band_rows):
+ *       out[m - band_row0, n] = cast( C[m,n] + sum_{j<n_peers} fp32(peers[j][m - band_row0, n]) + [bias[n]] )
+ *   for rows m outside the band, if c_full != NULL:   c_full[m, n] = bf16(C[m,n])
+ * A: element (m,k) at A[m*lda_m + k*lda_k]; lda_k must be 1.
+ * B: element (k,n) at B[k*ldb_k + n*ldb_n]; either ldb_n == 1 (row-major B)
+ *    or ldb_k == 1 (B transposed-contiguous, "NT").
+ * peers: n_peers contiguous [band_rows, N] bf16 matrices, peers_stride elements apart
+ *        (NULL with n_peers == 0 for a plain GEMM).  bias: [N] bf16 or NULL.
+ * out: [band_rows, N], row stride N; bf16, or fp32 when out_is_fp32 != 0.
+ * c_full: [M, N] bf16, row stride N, or NULL.
+ * tile_pivot: row offset (in rows) by which the order of M tiles is rotated;
+ *        changes scheduling only, never the result.
+ * Requirements: K % 8 == 0, N % 8 == 0, leading strides % 8 == 0, pointers
+ * 16-byte aligned, 0 <= band_row0, band_row0 + band_rows <= M.
+ *
+ * Replaces
+ *   kraken/fused/gemm_one_shot_all_reduce_fused.py:56-99   (band = all rows)
+ *   kraken/fused/gemm_reduce_scatter_fused.py:63-72,102-145 (band = this rank's M/W rows)
+ *   kraken/fused/all_gather_matmul.py:87-123               (n_peers = 0, tile_pivot = rank*m)
+ */
+int kr_gemm_reduce_bf16(const void* A, int64_t lda_m, int64_t lda_k,
+                        const void* B, int64_t ldb_k, int64_t ldb_n,
+                        int64_t M, int64_t N, int64_t K,
+                        const void* peers, int n_peers, int64_t peers_stride,
+                        const void* bias,
+                        int64_t band_row0, int64_t band_rows,
+                        void* c_full, void* out, int out_is_fp32,
+                        int64_t tile_pivot, void* stream);
+
+/*
+ * Tile reduce of the copy-engine reduce-scatter variant: `in` is [W*rows, N]
+ * bf16 (band r holds what rank r pushed), and
+ *   out[m, n] = sum_{i=0..W-1} in[((i + rank + 1) % W) * rows + m, n]
+ * accumulated in rotated order starting at rank+1.  acc_bf16 != 0 rounds the
+ * running sum to bf16 after every add (what the reference does); 0 keeps fp32.
+ * Replaces kraken/fused/gemm_reduce_scatter_ce_persistent.py:245-281.
+ */
+int kr_reduce_rotated_bf16(const void* in, int W, int64_t rows, int64_t N, int rank,
+                           int acc_bf16, void* out, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* KRAKEN_AMD_H */

@@ -1,0 +1,118 @@
+"""ctypes binding of libkraken_amd.so (the C ABI in include/kraken_amd.h)."""
+from __future__ import annotations
+
+import ctypes
+from ctypes import c_char_p, c_float, c_int, c_int64, c_void_p
+from pathlib import Path
+
+import torch
+
+LIB_PATH = Path(__file__).resolve().parent / "lib" / "libkraken_amd.so"
+
+# negative return codes of the library (include/kraken_amd.h)
+KR_OK = 0
+KR_ERR_NULL_POINTER = -1
+KR_ERR_ALIGNMENT = -2
+KR_ERR_NUMEL_MOD8 = -3
+KR_ERR_BAD_DIM = -4
+KR_ERR_WORLD_SIZE = -5
+KR_ERR_BIAS_SHAPE = -6
+KR_ERR_ROW_TOO_LONG = -7
+KR_ERR_BAND = -8
+KR_ERR_LAYOUT = -9
+KR_ERR_STRIPE = -10
+
+_SIGNATURES = {
+    "kr_version": (c_int, []),
+    "kr_strerror": (c_char_p, [c_int]),
+    "kr_reduce_bf16": (
+        c_int,
+        [c_void_p, c_int, c_int64, c_int64, c_void_p, c_int64, c_int64, c_int, c_void_p, c_void_p],
+    ),
+    "kr_reduce_striped_bf16": (
+        c_int,
+        [c_void_p, c_int, c_int64, c_int64, c_void_p, c_int64, c_int, c_void_p, c_void_p],
+    ),
+    "kr_striped_share_numel": (c_int64, [c_int64, c_int, c_int64, c_int]),
+    "kr_reduce_rmsnorm_bf16": (
+        c_int,
+        [c_void_p, c_int, c_int64, c_int64, c_int64, c_void_p, c_int, c_void_p, c_float, c_void_p, c_void_p],
+    ),
+    "kr_rmsnorm_bf16": (c_int, [c_void_p, c_void_p, c_float, c_int64, c_int64, c_void_p, c_void_p]),
+    "kr_gemm_reduce_bf16": (
+        c_int,
+        [c_void_p, c_int64, c_int64, c_void_p, c_int64, c_int64, c_int64, c_int64, c_int64,
+         c_void_p, c_int, c_int64, c_void_p, c_int64, c_int64, c_void_p, c_void_p, c_int, c_int64, c_void_p],
+    ),
+    "kr_reduce_rotated_bf16": (c_int, [c_void_p, c_int, c_int64, c_int64, c_int, c_int, c_void_p, c_void_p]),
+}
+
+EXPORTS = tuple(_SIGNATURES)
+
+_lib = None
+
+
+class KrakenAmdError(RuntimeError):
+    """A HIP error reported by a kernel launch (positive return code)."""
+
+
+def load() -> ctypes.CDLL:
+    """Load libkraken_amd.so once; raise if it has not been built."""
+    global _lib
+    if _lib is None:
+        if not LIB_PATH.exists():
+            raise RuntimeError(
+                f"{LIB_PATH} is missing: build it with `python -m kraken_amd.build` "
+                "(kraken_amd has no CPU or PyTorch fallback)"
+            )
+        lib = ctypes.CDLL(str(LIB_PATH))
+        for name, (restype, argtypes) in _SIGNATURES.items():
+            fn = getattr(lib, name)
+            fn.restype = restype
+            fn.argtypes = argtypes
+        _lib = lib
+    return _lib
+
+
+def strerror(code: int) -> str:
+    return load().kr_strerror(int(code)).decode()
+
+
+def check(code: int, what: str) -> None:
+    """Map a library return code to the exception the reference would raise."""
+    if code == KR_OK:
+        return
+    msg = f"{what}: {strerror(code)} (code {code})"
+    if code > 0:
+        raise KrakenAmdError(msg)
+    if code in (KR_ERR_LAYOUT, KR_ERR_NULL_POINTER):
+        raise ValueError(msg)
+    raise AssertionError(msg)
+
+
+def require_device(*tensors: torch.Tensor | None) -> torch.device:
+    """All given tensors must live on one HIP device (no host fallback exists)."""
+    dev = None
+    for t in tensors:
+        if t is None:
+            continue
+        if not t.is_cuda:
+            raise RuntimeError(
+                "kraken_amd kernels run on a HIP device only; got a tensor on "
+                f"'{t.device}' (there is no CPU fallback)"
+            )
+        if dev is None:
+            dev = t.device
+        elif t.device != dev:
+            raise RuntimeError(f"tensors on different devices: {dev} and {t.device}")
+    if dev is None:
+        raise RuntimeError("no device tensor given")
+    return dev
+
+
+def ptr(t: torch.Tensor | None) -> int | None:
+    return None if t is None else t.data_ptr()
+
+
+def current_stream(dev: torch.device) -> int:
+    return torch.cuda.current_stream(dev).cuda_stream

@@ -1,0 +1,95 @@
+// Shared device helpers for the gfx950 kernels: bf16 <-> fp32 packing, 128-bit
+// vector access, wave64 reductions, host-side argument checks.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/kraken_amd.h"
+
+namespace kr {
+
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+
+constexpr int kWave = 64;
+
+// ---- bf16 packing ---------------------------------------------------------
+// A 32-bit word holds two bf16: element 2j in the low half, 2j+1 in the high half.
+__device__ __forceinline__ float bf16_lo(uint32_t w) { return __builtin_bit_cast(float, w << 16); }
+__device__ __forceinline__ float bf16_hi(uint32_t w) { return __builtin_bit_cast(float, w & 0xffff0000u); }
+
+// fp32 pair -> packed bf16 pair, round-to-nearest-even (v_cvt_pk_bf16_f32 on gfx950).
+__device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) {
+    bf16x2 p;
+    p.x = (__bf16)lo;
+    p.y = (__bf16)hi;
+    return __builtin_bit_cast(uint32_t, p);
+}
+
+// 8 bf16 (one 128-bit vector) <-> 8 fp32
+__device__ __forceinline__ void unpack8(const u32x4 v, float (&f)[8]) {
+    f[0] = bf16_lo(v.x); f[1] = bf16_hi(v.x);
+    f[2] = bf16_lo(v.y); f[3] = bf16_hi(v.y);
+    f[4] = bf16_lo(v.z); f[5] = bf16_hi(v.z);
+    f[6] = bf16_lo(v.w); f[7] = bf16_hi(v.w);
+}
+__device__ __forceinline__ void zero8(float (&f)[8]) {
+#pragma unroll
+    for (int j = 0; j < 8; ++j) f[j] = 0.0f;
+}
+// column (in 128-bit vectors) of flat vector index i in rows of d vectors
+__device__ __forceinline__ uint32_t mod_vec(int64_t i, uint32_t d) {
+    return (uint64_t)i <= 0xffffffffull ? (uint32_t)i % d : (uint32_t)((uint64_t)i % d);
+}
+__device__ __forceinline__ void add8(const u32x4 v, float (&f)[8]) {
+    f[0] += bf16_lo(v.x); f[1] += bf16_hi(v.x);
+    f[2] += bf16_lo(v.y); f[3] += bf16_hi(v.y);
+    f[4] += bf16_lo(v.z); f[5] += bf16_hi(v.z);
+    f[6] += bf16_lo(v.w); f[7] += bf16_hi(v.w);
+}
+__device__ __forceinline__ u32x4 pack8(const float (&f)[8]) {
+    u32x4 v;
+    v.x = pack_bf16(f[0], f[1]);
+    v.y = pack_bf16(f[2], f[3]);
+    v.z = pack_bf16(f[4], f[5]);
+    v.w = pack_bf16(f[6], f[7]);
+    return v;
+}
+
+// Streaming 128-bit accesses: every input byte of the reduce paths is used
+// exactly once, so loads and stores carry the non-temporal hint.
+__device__ __forceinline__ u32x4 ld_stream(const u32x4* p) { return __builtin_nontemporal_load(p); }
+__device__ __forceinline__ void st_stream(u32x4* p, u32x4 v) { __builtin_nontemporal_store(v, p); }
+
+// ---- wave64 sum -------------------------------------------------------------
+// Sum over the 64 lanes of a wavefront; every lane returns the total.  The
+// first four steps stay inside a row of 16 lanes and use DPP lane permutes
+// (no LDS traffic); the four row totals are then combined through readlane.
+template <int CTRL>
+__device__ __forceinline__ float dpp_f32(float v) {
+    return __builtin_bit_cast(
+        float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, false));
+}
+__device__ __forceinline__ float wave_sum(float v) {
+    v += dpp_f32<0xB1>(v);   // quad_perm [1,0,3,2]
+    v += dpp_f32<0x4E>(v);   // quad_perm [2,3,0,1]
+    v += dpp_f32<0x141>(v);  // row_half_mirror
+    v += dpp_f32<0x140>(v);  // row_mirror
+    const int b = __builtin_bit_cast(int, v);
+    const float r0 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(b, 0));
+    const float r1 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(b, 16));
+    const float r2 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(b, 32));
+    const float r3 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(b, 48));
+    return (r0 + r1) + (r2 + r3);
+}
+
+// ---- host-side checks -------------------------------------------------------
+static inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+}  // namespace kr

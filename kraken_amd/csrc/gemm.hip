@@ -1,0 +1,388 @@
+// bf16 GEMM on the gfx950 matrix cores with a fused reduce(+bias) epilogue.
+//
+//   C = A[M,K] @ B[K,N]                      (fp32 accumulate, v_mfma_f32_32x32x16_bf16)
+//   out  = C[band] + sum_j peers[j] + bias   (rows of the band; one store, no C round trip)
+//   c_full[rows outside the band] = bf16(C)
+//
+// Workgroup tile BM x BN x 64, WM x WN wavefronts, each owning a
+// (BM/WM) x (BN/WN) block of C as 32x32 MFMA accumulators.  A and B tiles are
+// staged in LDS as [row][64 k] bf16 (128-byte rows) with the 16-byte chunks of
+// a row XOR-swizzled by the row index, so that the 128-bit fragment reads of 8
+// consecutive rows land in 8 different bank groups.  Two LDS stages: the
+// global loads of k-step t+1 are issued before the MFMAs of step t and written
+// to the other stage afterwards (one workgroup barrier per k-step).
+// Row-major B ([K,N], N contiguous) is transposed on its way into LDS: a
+// thread loads an 8(k) x 8(n) block with eight 128-bit loads, transposes it in
+// registers with byte permutes and writes eight 128-bit [n][8 k] chunks.
+// Epilogue: accumulators go through a per-wave LDS patch to turn the MFMA
+// layout into row-contiguous 8-element vectors, so peers, bias and output are
+// all moved with 128-bit accesses covering whole 256-byte row segments.
+#include <stdlib.h>
+
+#include "common.h"
+
+namespace kr {
+
+struct GemmArgs {
+    const uint16_t* A;
+    const uint16_t* B;
+    int64_t lda;   // elements between rows of A (k is contiguous)
+    int64_t ldb;   // NT: elements between n-rows of B^T; NN: elements between k-rows of B
+    int M, N, K;
+    const uint16_t* peers;
+    int n_peers;
+    int64_t peers_stride;
+    const uint16_t* bias;
+    int band_row0, band_rows;
+    uint16_t* c_full;
+    void* out;
+    int out_is_fp32;
+    int pivot_tiles;   // rotation of the M-tile order
+    int tiles_m, tiles_n;
+};
+
+constexpr int BK = 64;            // k extent of one LDS stage
+constexpr int kRowBytes = BK * 2; // 128-byte LDS rows
+constexpr int kGroupM = 4;        // M tiles per scheduling group
+constexpr int kXcds = 8;
+
+// 16-byte chunk swizzle inside a 128-byte LDS row
+__device__ __forceinline__ int swz(int row, int chunk) { return chunk ^ ((row ^ (row >> 3)) & 7); }
+
+__device__ __forceinline__ uint32_t perm_lo(uint32_t hi_src, uint32_t lo_src) {
+    // {lo16(hi_src), lo16(lo_src)}
+    return __builtin_amdgcn_perm(hi_src, lo_src, 0x05040100u);
+}
+__device__ __forceinline__ uint32_t perm_hi(uint32_t hi_src, uint32_t lo_src) {
+    // {hi16(hi_src), hi16(lo_src)}
+    return __builtin_amdgcn_perm(hi_src, lo_src, 0x07060302u);
+}
+
+template <int BM, int BN, int WM, int WN, bool B_NT, bool EVEN>
+__global__ __launch_bounds__(WM* WN * 64) void gemm_reduce_kernel(const GemmArgs g) {
+    constexpr int T = WM * WN * 64;
+    constexpr int WTM = BM / WM, WTN = BN / WN;   // wave tile
+    constexpr int TM = WTM / 32, TN = WTN / 32;   // 32x32 MFMA blocks per wave
+    constexpr int A_STAGE = BM * kRowBytes, B_STAGE = BN * kRowBytes;
+    constexpr int STAGE = A_STAGE + B_STAGE;
+    constexpr int A_ITERS = BM * 8 / T;           // 16-byte chunks per thread per stage
+    constexpr int B_ITERS_NT = BN * 8 / T;
+    constexpr int B_BLOCKS = BN / T > 0 ? BN / T : 1;  // NN: 8x8 blocks per thread per stage
+    static_assert(BM % (WM * 32) == 0 && BN % (WN * 32) == 0, "wave tile must be a multiple of 32");
+    static_assert((BM * 8) % T == 0 && (BN * 8) % T == 0 && (BN % T == 0 || BN < T), "load split");
+    // epilogue patch: 32 rows x WTN fp32 per wave, rows padded by 4 floats
+    constexpr int EP_LD = WTN + 4;
+    constexpr int EP_WAVE = 32 * EP_LD * 4;
+    static_assert(EP_WAVE * WM * WN <= 2 * STAGE, "epilogue patch must fit in the pipeline LDS");
+
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = tid >> 6;
+    const int wm = wave / WN, wn = wave % WN;
+
+    // ---- tile schedule: XCD-contiguous, grouped along M, rotated by the pivot
+    int pid = blockIdx.x;
+    const int ntiles = g.tiles_m * g.tiles_n;
+    if (ntiles % kXcds == 0) pid = (pid % kXcds) * (ntiles / kXcds) + pid / kXcds;
+    const int per_group = kGroupM * g.tiles_n;
+    const int group = pid / per_group;
+    const int first_m = group * kGroupM;
+    const int gsz = min(g.tiles_m - first_m, kGroupM);
+    int tile_m = first_m + (pid % per_group) % gsz;
+    const int tile_n = (pid % per_group) / gsz;
+    tile_m += g.pivot_tiles;
+    if (tile_m >= g.tiles_m) tile_m -= g.tiles_m;
+    const int m0 = tile_m * BM, n0 = tile_n * BN;
+
+    // ---- global -> register staging ------------------------------------------
+    u32x4 a_reg[A_ITERS];
+    u32x4 b_reg[B_NT ? B_ITERS_NT : B_BLOCKS * 8];
+
+    auto load_a = [&](int k0) {
+#pragma unroll
+        for (int i = 0; i < A_ITERS; ++i) {
+            const int c = i * T + tid;
+            const int row = c >> 3, kc = c & 7;
+            int m = m0 + row;
+            const int k = k0 + kc * 8;
+            if (EVEN) {
+                a_reg[i] = *(const u32x4*)(g.A + (int64_t)m * g.lda + k);
+            } else {
+                m = min(m, g.M - 1);
+                a_reg[i] = k < g.K ? *(const u32x4*)(g.A + (int64_t)m * g.lda + k) : u32x4{0, 0, 0, 0};
+            }
+        }
+    };
+    auto load_b = [&](int k0) {
+        if (B_NT) {
+#pragma unroll
+            for (int i = 0; i < B_ITERS_NT; ++i) {
+                const int c = i * T + tid;
+                const int row = c >> 3, kc = c & 7;
+                int n = n0 + row;
+                const int k = k0 + kc * 8;
+                if (EVEN) {
+                    b_reg[i] = *(const u32x4*)(g.B + (int64_t)n * g.ldb + k);
+                } else {
+                    n = min(n, g.N - 1);
+                    b_reg[i] = k < g.K ? *(const u32x4*)(g.B + (int64_t)n * g.ldb + k) : u32x4{0, 0, 0, 0};
+                }
+            }
+        } else {
+#pragma unroll
+            for (int i = 0; i < B_BLOCKS; ++i) {
+                const int blk = i * T + tid;
+                const int nc = blk % (BN / 8), kg = blk / (BN / 8);
+                if (BN < T && kg >= 8) continue;  // more threads than 8x8 blocks
+                int n = n0 + nc * 8;
+                if (!EVEN) n = min(n, g.N - 8);
+#pragma unroll
+                for (int j = 0; j < 8; ++j) {
+                    const int k = k0 + kg * 8 + j;
+                    if (EVEN) {
+                        b_reg[i * 8 + j] = *(const u32x4*)(g.B + (int64_t)k * g.ldb + n);
+                    } else {
+                        b_reg[i * 8 + j] =
+                            k < g.K ? *(const u32x4*)(g.B + (int64_t)k * g.ldb + n) : u32x4{0, 0, 0, 0};
+                    }
+                }
+            }
+        }
+    };
+    auto store_stage = [&](int stage) {
+        unsigned char* As = smem + stage * STAGE;
+        unsigned char* Bs = As + A_STAGE;
+#pragma unroll
+        for (int i = 0; i < A_ITERS; ++i) {
+            const int c = i * T + tid;
+            const int row = c >> 3, kc = c & 7;
+            *(u32x4*)(As + row * kRowBytes + swz(row, kc) * 16) = a_reg[i];
+        }
+        if (B_NT) {
+#pragma unroll
+            for (int i = 0; i < B_ITERS_NT; ++i) {
+                const int c = i * T + tid;
+                const int row = c >> 3, kc = c & 7;
+                *(u32x4*)(Bs + row * kRowBytes + swz(row, kc) * 16) = b_reg[i];
+            }
+        } else {
+#pragma unroll
+            for (int i = 0; i < B_BLOCKS; ++i) {
+                const int blk = i * T + tid;
+                const int nc = blk % (BN / 8), kg = blk / (BN / 8);
+                if (BN < T && kg >= 8) continue;
+                // b_reg[i*8 + j] holds row k = kg*8 + j, columns nc*8 .. nc*8+7 (two per word)
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {      // word q = columns 2q, 2q+1
+                    u32x4 even, odd;               // [n = 2q][k 0..7], [n = 2q+1][k 0..7]
+                    even.x = perm_lo(b_reg[i * 8 + 1][q], b_reg[i * 8 + 0][q]);
+                    even.y = perm_lo(b_reg[i * 8 + 3][q], b_reg[i * 8 + 2][q]);
+                    even.z = perm_lo(b_reg[i * 8 + 5][q], b_reg[i * 8 + 4][q]);
+                    even.w = perm_lo(b_reg[i * 8 + 7][q], b_reg[i * 8 + 6][q]);
+                    odd.x = perm_hi(b_reg[i * 8 + 1][q], b_reg[i * 8 + 0][q]);
+                    odd.y = perm_hi(b_reg[i * 8 + 3][q], b_reg[i * 8 + 2][q]);
+                    odd.z = perm_hi(b_reg[i * 8 + 5][q], b_reg[i * 8 + 4][q]);
+                    odd.w = perm_hi(b_reg[i * 8 + 7][q], b_reg[i * 8 + 6][q]);
+                    const int r0 = nc * 8 + 2 * q, r1 = r0 + 1;
+                    *(u32x4*)(Bs + r0 * kRowBytes + swz(r0, kg) * 16) = even;
+                    *(u32x4*)(Bs + r1 * kRowBytes + swz(r1, kg) * 16) = odd;
+                }
+            }
+        }
+    };
+
+    // ---- main loop ----------------------------------------------------------------
+    f32x16 acc[TM][TN];
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
+
+    const int kt_total = (g.K + BK - 1) / BK;
+    load_a(0);
+    load_b(0);
+    store_stage(0);
+    __syncthreads();
+
+    const int frag_row = lane & 31;   // row (A) / column (B) inside a 32x32 block
+    const int frag_kc = lane >> 5;    // which 8-wide k chunk of the 16-wide MFMA step
+
+    for (int kt = 0; kt < kt_total; ++kt) {
+        const int cur = kt & 1;
+        const bool more = kt + 1 < kt_total;
+        if (more) {
+            load_a((kt + 1) * BK);
+            load_b((kt + 1) * BK);
+        }
+        const unsigned char* As = smem + cur * STAGE;
+        const unsigned char* Bs = As + A_STAGE;
+#pragma unroll
+        for (int ks = 0; ks < BK / 16; ++ks) {
+            bf16x8 af[TM], bfr[TN];
+#pragma unroll
+            for (int i = 0; i < TM; ++i) {
+                const int row = wm * WTM + i * 32 + frag_row;
+                af[i] = *(const bf16x8*)(As + row * kRowBytes + swz(row, ks * 2 + frag_kc) * 16);
+            }
+#pragma unroll
+            for (int j = 0; j < TN; ++j) {
+                const int row = wn * WTN + j * 32 + frag_row;
+                bfr[j] = *(const bf16x8*)(Bs + row * kRowBytes + swz(row, ks * 2 + frag_kc) * 16);
+            }
+#pragma unroll
+            for (int i = 0; i < TM; ++i)
+#pragma unroll
+                for (int j = 0; j < TN; ++j)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[i], bfr[j], acc[i][j], 0, 0, 0);
+        }
+        if (more) store_stage(cur ^ 1);
+        __syncthreads();
+    }
+
+    // ---- epilogue -------------------------------------------------------------------
+    // After the last barrier no wave reads the pipeline stages any more.
+    float* patch = (float*)(smem + wave * EP_WAVE);
+    constexpr int CPR = WTN / 8;            // 8-element chunks per patch row
+    constexpr int EP_ITERS = 32 * CPR / 64; // chunks per lane per 32-row slab
+    const int band_lo = g.band_row0, band_hi = g.band_row0 + g.band_rows;
+
+#pragma unroll
+    for (int i = 0; i < TM; ++i) {
+        // MFMA layout: lane holds column (lane & 31); register v is row 8*(v/4) + 4*(lane>>5) + v%4
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+                const int r = 8 * (v >> 2) + 4 * (lane >> 5) + (v & 3);
+                patch[r * EP_LD + j * 32 + (lane & 31)] = acc[i][j][v];
+            }
+        __syncthreads();
+#pragma unroll
+        for (int it = 0; it < EP_ITERS; ++it) {
+            const int c = it * 64 + lane;
+            const int r = c / CPR, cc = c % CPR;
+            const int m = m0 + wm * WTM + i * 32 + r;
+            const int n = n0 + wn * WTN + cc * 8;
+            if (!EVEN && (m >= g.M || n >= g.N)) continue;
+            float f[8];
+            const f32x4 lo = *(const f32x4*)(patch + r * EP_LD + cc * 8);
+            const f32x4 hi = *(const f32x4*)(patch + r * EP_LD + cc * 8 + 4);
+            f[0] = lo.x; f[1] = lo.y; f[2] = lo.z; f[3] = lo.w;
+            f[4] = hi.x; f[5] = hi.y; f[6] = hi.z; f[7] = hi.w;
+            if (m >= band_lo && m < band_hi) {
+                const int64_t off = (int64_t)(m - band_lo) * g.N + n;
+                for (int p = 0; p < g.n_peers; ++p)
+                    add8(ld_stream((const u32x4*)(g.peers + p * g.peers_stride + off)), f);
+                if (g.bias != nullptr) add8(*(const u32x4*)(g.bias + n), f);
+                if (g.out_is_fp32) {
+                    float* o = (float*)g.out + off;
+                    *(f32x4*)o = f32x4{f[0], f[1], f[2], f[3]};
+                    *(f32x4*)(o + 4) = f32x4{f[4], f[5], f[6], f[7]};
+                } else {
+                    st_stream((u32x4*)((uint16_t*)g.out + off), pack8(f));
+                }
+            } else if (g.c_full != nullptr) {
+                st_stream((u32x4*)(g.c_full + (int64_t)m * g.N + n), pack8(f));
+            }
+        }
+        __syncthreads();
+    }
+}
+
+template <int BM, int BN, int WM, int WN>
+static hipError_t launch_gemm(const GemmArgs& g, bool b_nt, bool even, hipStream_t st) {
+    constexpr int T = WM * WN * 64;
+    constexpr int LDS = 2 * (BM + BN) * kRowBytes;
+    const dim3 grid((unsigned)(g.tiles_m * g.tiles_n)), block(T);
+#define KR_LAUNCH(NT, EV)                                                                             \
+    do {                                                                                              \
+        auto kfn = gemm_reduce_kernel<BM, BN, WM, WN, NT, EV>;                                        \
+        static bool lds_opt_in = false; /* benign race: the attribute call is idempotent */          \
+        if (!lds_opt_in) {                                                                            \
+            hipError_t e = hipFuncSetAttribute((const void*)kfn,                                      \
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, LDS);      \
+            if (e != hipSuccess) return e;                                                            \
+            lds_opt_in = true;                                                                        \
+        }                                                                                             \
+        hipLaunchKernelGGL(kfn, grid, block, LDS, st, g);                                             \
+    } while (0)
+    if (b_nt) {
+        if (even) KR_LAUNCH(true, true); else KR_LAUNCH(true, false);
+    } else {
+        if (even) KR_LAUNCH(false, true); else KR_LAUNCH(false, false);
+    }
+#undef KR_LAUNCH
+    return hipGetLastError();
+}
+
+}  // namespace kr
+
+using namespace kr;
+
+extern "C" int kr_gemm_reduce_bf16(const void* A, int64_t lda_m, int64_t lda_k, const void* B, int64_t ldb_k,
+                                   int64_t ldb_n, int64_t M, int64_t N, int64_t K, const void* peers,
+                                   int n_peers, int64_t peers_stride, const void* bias, int64_t band_row0,
+                                   int64_t band_rows, void* c_full, void* out, int out_is_fp32,
+                                   int64_t tile_pivot, void* stream) {
+    if (M < 0 || N < 0 || K < 0 || M > 0x7fffffffLL || N > 0x7fffffffLL || K > 0x7fffffffLL)
+        return KR_ERR_BAD_DIM;
+    if (n_peers < 0 || n_peers >= KR_MAX_WORLD) return KR_ERR_WORLD_SIZE;
+    if (band_row0 < 0 || band_rows < 0 || band_row0 + band_rows > M) return KR_ERR_BAND;
+    if (K % 8 != 0 || N % 8 != 0) return KR_ERR_NUMEL_MOD8;
+    if (M == 0 || N == 0) return KR_OK;
+    if (K == 0) return KR_ERR_BAD_DIM;
+    if (A == nullptr || B == nullptr) return KR_ERR_NULL_POINTER;
+    if (band_rows > 0 && out == nullptr) return KR_ERR_NULL_POINTER;
+    if (n_peers > 0 && peers == nullptr) return KR_ERR_NULL_POINTER;
+    if (lda_k != 1) return KR_ERR_LAYOUT;
+    const bool b_nt = (ldb_k == 1 && (ldb_n != 1 || N == 1));
+    if (!b_nt && ldb_n != 1) return KR_ERR_LAYOUT;
+    const int64_t ldb = b_nt ? ldb_n : ldb_k;
+    if (lda_m < K || (b_nt ? ldb < K : ldb < N)) return KR_ERR_LAYOUT;
+    if (lda_m % 8 != 0 || ldb % 8 != 0 || peers_stride % 8 != 0) return KR_ERR_ALIGNMENT;
+    if (!aligned16(A) || !aligned16(B) || !aligned16(peers) || !aligned16(bias) || !aligned16(c_full) ||
+        !aligned16(out))
+        return KR_ERR_ALIGNMENT;
+    if (n_peers > 0 && peers_stride < band_rows * N) return KR_ERR_BAD_DIM;
+
+    GemmArgs g;
+    g.A = (const uint16_t*)A;
+    g.B = (const uint16_t*)B;
+    g.lda = lda_m;
+    g.ldb = ldb;
+    g.M = (int)M; g.N = (int)N; g.K = (int)K;
+    g.peers = (const uint16_t*)peers;
+    g.n_peers = n_peers;
+    g.peers_stride = peers_stride;
+    g.bias = (const uint16_t*)bias;
+    g.band_row0 = (int)band_row0;
+    g.band_rows = (int)band_rows;
+    g.c_full = (uint16_t*)c_full;
+    g.out = out;
+    g.out_is_fp32 = out_is_fp32;
+
+    // Tile choice: the 256x256 tile (4 waves x 128x128) has the highest MFMA
+    // work per LDS/HBM byte; it needs enough tiles to fill 256 CUs and a K loop
+    // long enough to amortise its epilogue.  Otherwise 128x128 tiles, several
+    // of which share a CU so that one tile's epilogue overlaps another's MFMAs.
+    bool big = (M % 256 == 0 && N % 256 == 0 && K % BK == 0 && (M / 256) * (N / 256) >= 256 && K >= 2048);
+    // KRAKEN_AMD_GEMM_TILE=128|256 overrides the choice (testing and tuning)
+    if (const char* t = getenv("KRAKEN_AMD_GEMM_TILE")) {
+        if (t[0] == '1') big = false;
+        if (t[0] == '2') big = true;
+    }
+    const int bm = big ? 256 : 128, bn = big ? 256 : 128;
+    g.tiles_m = (int)((M + bm - 1) / bm);
+    g.tiles_n = (int)((N + bn - 1) / bn);
+    if ((int64_t)g.tiles_m * g.tiles_n > 0x7fffffffLL) return KR_ERR_BAD_DIM;
+    int64_t pt = tile_pivot / bm;
+    g.pivot_tiles = (int)(((pt % g.tiles_m) + g.tiles_m) % g.tiles_m);
+    const bool even = (M % bm == 0 && N % bn == 0 && K % BK == 0);
+    hipError_t e = big ? launch_gemm<256, 256, 2, 2>(g, b_nt, even, (hipStream_t)stream)
+                       : launch_gemm<128, 128, 2, 2>(g, b_nt, even, (hipStream_t)stream);
+    return (int)e;
+}

@@ -1,0 +1,266 @@
+// W-way elementwise reduce (+bias) over the W slices of a stacked bf16 tensor.
+//
+// HBM-bound: per output vector of 8 elements the kernel reads W*16 B (+16 B of
+// bias) and writes 16 B, i.e. (W+1)*2 bytes per element.  Every thread owns
+// kUnroll 128-bit vectors that are kThreads vectors apart, so each wave-level
+// load covers 1 KiB of consecutive addresses, and all W*kUnroll loads of a
+// thread are issued before the first add (the adds keep the fixed order
+// bias?, slice 0, 1, ... W-1, so the sum is reproducible bit for bit).
+#include "common.h"
+
+namespace kr {
+
+constexpr int kThreads = 256;
+constexpr int kUnroll = 2;
+
+enum BiasMode { kNoBias = 0, kFullBias = 1, kVectorBias = 2 };
+
+// WT > 0: W known at compile time (loop fully unrolled); WT == 0: run-time W.
+template <int WT, int BIAS, bool BIAS_FIRST>
+__global__ __launch_bounds__(kThreads) void reduce_kernel(
+    const u32x4* __restrict__ stack, int w_rt, int64_t slice_stride_v, int64_t nvec,
+    const u32x4* __restrict__ bias, uint32_t d_vec, u32x4* __restrict__ out) {
+    const int W = WT > 0 ? WT : w_rt;
+    const int64_t base = (int64_t)blockIdx.x * (kThreads * kUnroll) + threadIdx.x;
+
+    if (base + (int64_t)(kUnroll - 1) * kThreads < nvec) {
+        // full block: no bounds checks
+        float acc[kUnroll][8];
+        u32x4 bv[kUnroll];
+        if (BIAS != kNoBias) {
+#pragma unroll
+            for (int u = 0; u < kUnroll; ++u) {
+                const int64_t i = base + (int64_t)u * kThreads;
+                bv[u] = BIAS == kFullBias ? ld_stream(bias + i) : bias[mod_vec(i, d_vec)];
+            }
+        }
+        if (WT > 0) {
+            u32x4 v[WT > 0 ? WT : 1][kUnroll];
+#pragma unroll
+            for (int r = 0; r < WT; ++r)
+#pragma unroll
+                for (int u = 0; u < kUnroll; ++u)
+                    v[r][u] = ld_stream(stack + r * slice_stride_v + base + (int64_t)u * kThreads);
+#pragma unroll
+            for (int u = 0; u < kUnroll; ++u) {
+                if (BIAS != kNoBias && BIAS_FIRST) {
+                    unpack8(bv[u], acc[u]);
+                    add8(v[0][u], acc[u]);
+                } else {
+                    zero8(acc[u]);  // acc = 0.0f, then += slice 0 (keeps the sign of a -0.0 sum as the reference has it)
+                    add8(v[0][u], acc[u]);
+                }
+#pragma unroll
+                for (int r = 1; r < WT; ++r) add8(v[r][u], acc[u]);
+            }
+        } else {
+#pragma unroll
+            for (int u = 0; u < kUnroll; ++u) {
+                const u32x4* p = stack + base + (int64_t)u * kThreads;
+                if (BIAS != kNoBias && BIAS_FIRST) {
+                    unpack8(bv[u], acc[u]);
+                    add8(ld_stream(p), acc[u]);
+                } else {
+                    zero8(acc[u]);
+                    add8(ld_stream(p), acc[u]);
+                }
+                for (int r = 1; r < W; ++r) add8(ld_stream(p + r * slice_stride_v), acc[u]);
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < kUnroll; ++u) {
+            if (BIAS != kNoBias && !BIAS_FIRST) add8(bv[u], acc[u]);
+            st_stream(out + base + (int64_t)u * kThreads, pack8(acc[u]));
+        }
+    } else {
+        // ragged last block
+        for (int u = 0; u < kUnroll; ++u) {
+            const int64_t i = base + (int64_t)u * kThreads;
+            if (i >= nvec) break;
+            float acc[8];
+            u32x4 bv = {0, 0, 0, 0};
+            if (BIAS != kNoBias) bv = BIAS == kFullBias ? bias[i] : bias[mod_vec(i, d_vec)];
+            const u32x4* p = stack + i;
+            if (BIAS != kNoBias && BIAS_FIRST) {
+                unpack8(bv, acc);
+                add8(p[0], acc);
+            } else {
+                zero8(acc);
+                add8(p[0], acc);
+            }
+            for (int r = 1; r < W; ++r) add8(p[r * slice_stride_v], acc);
+            if (BIAS != kNoBias && !BIAS_FIRST) add8(bv, acc);
+            out[i] = pack8(acc);
+        }
+    }
+}
+
+// Striped ownership: output vector j (compact) comes from input vector
+//   (j / blk_v) * blk_v * W + rank * blk_v + (j % blk_v).
+__global__ __launch_bounds__(kThreads) void reduce_striped_kernel(
+    const u32x4* __restrict__ stack, int W, int64_t slice_stride_v, int64_t share_nvec,
+    const u32x4* __restrict__ bias, uint32_t blk_v, int rank, u32x4* __restrict__ out) {
+    const int64_t j = (int64_t)blockIdx.x * kThreads + threadIdx.x;
+    if (j >= share_nvec) return;
+    const int64_t stripe = j / blk_v;
+    const int64_t i = (stripe * W + rank) * blk_v + (j - stripe * blk_v);
+    float acc[8];
+    const u32x4* p = stack + i;
+    zero8(acc);
+    add8(ld_stream(p), acc);
+    for (int r = 1; r < W; ++r) add8(ld_stream(p + r * slice_stride_v), acc);
+    if (bias != nullptr) add8(ld_stream(bias + i), acc);
+    st_stream(out + j, pack8(acc));
+}
+
+// Rotated-order tile reduce of the copy-engine reduce-scatter variant:
+// out[v] = sum_i in[((i + rank + 1) % W) * band_v + v], optionally rounding
+// the running sum to bf16 after every add.
+template <bool ACC_BF16>
+__global__ __launch_bounds__(kThreads) void reduce_rotated_kernel(
+    const u32x4* __restrict__ in, int W, int64_t band_v, int rank, u32x4* __restrict__ out) {
+    const int64_t v = (int64_t)blockIdx.x * kThreads + threadIdx.x;
+    if (v >= band_v) return;
+    float acc[8];
+    int cur = (rank + 1) % W;
+    unpack8(ld_stream(in + cur * band_v + v), acc);
+    for (int i = 1; i < W; ++i) {
+        cur = cur + 1 == W ? 0 : cur + 1;
+        add8(ld_stream(in + cur * band_v + v), acc);
+        if (ACC_BF16) unpack8(pack8(acc), acc);
+    }
+    st_stream(out + v, pack8(acc));
+}
+
+template <int WT, int BIAS>
+static hipError_t launch_reduce2(bool bias_first, dim3 grid, hipStream_t s, const u32x4* stack, int W,
+                                 int64_t ssv, int64_t nvec, const u32x4* bias, uint32_t d_vec, u32x4* out) {
+    if (bias_first)
+        hipLaunchKernelGGL((reduce_kernel<WT, BIAS, true>), grid, dim3(kThreads), 0, s, stack, W, ssv, nvec,
+                           bias, d_vec, out);
+    else
+        hipLaunchKernelGGL((reduce_kernel<WT, BIAS, false>), grid, dim3(kThreads), 0, s, stack, W, ssv, nvec,
+                           bias, d_vec, out);
+    return hipGetLastError();
+}
+
+template <int WT>
+static hipError_t launch_reduce1(int mode, bool bias_first, dim3 grid, hipStream_t s, const u32x4* stack,
+                                 int W, int64_t ssv, int64_t nvec, const u32x4* bias, uint32_t d_vec,
+                                 u32x4* out) {
+    switch (mode) {
+        case kNoBias:
+            // without a bias both orders are the same kernel
+            return launch_reduce2<WT, kNoBias>(true, grid, s, stack, W, ssv, nvec, bias, d_vec, out);
+        case kFullBias:
+            return launch_reduce2<WT, kFullBias>(bias_first, grid, s, stack, W, ssv, nvec, bias, d_vec, out);
+        default:
+            return launch_reduce2<WT, kVectorBias>(bias_first, grid, s, stack, W, ssv, nvec, bias, d_vec, out);
+    }
+}
+
+}  // namespace kr
+
+using namespace kr;
+
+static int check_reduce_common(const void* stack, int W, int64_t slice_stride, int64_t numel, const void* out) {
+    if (W < 1 || W > KR_MAX_WORLD) return KR_ERR_WORLD_SIZE;
+    if (numel < 0) return KR_ERR_BAD_DIM;
+    if (numel % 8 != 0) return KR_ERR_NUMEL_MOD8;
+    if (numel == 0) return KR_OK;
+    if (stack == nullptr || out == nullptr) return KR_ERR_NULL_POINTER;
+    if (!aligned16(stack) || !aligned16(out) || slice_stride % 8 != 0) return KR_ERR_ALIGNMENT;
+    if (slice_stride < 0) return KR_ERR_BAD_DIM;
+    return KR_OK;
+}
+
+extern "C" int kr_reduce_bf16(const void* stack, int W, int64_t slice_stride, int64_t numel, const void* bias,
+                              int64_t bias_numel, int64_t D, int bias_first, void* out, void* stream) {
+    int rc = check_reduce_common(stack, W, slice_stride, numel, out);
+    if (rc != KR_OK) return rc;
+    int mode = kNoBias;
+    if (bias != nullptr) {
+        if (!aligned16(bias)) return KR_ERR_ALIGNMENT;
+        if (bias_numel == numel) {
+            mode = kFullBias;
+        } else if (D > 0 && bias_numel == D && D % 8 == 0 && numel % D == 0) {
+            mode = kVectorBias;
+        } else {
+            return KR_ERR_BIAS_SHAPE;
+        }
+    }
+    if (numel == 0) return KR_OK;
+    const int64_t nvec = numel / 8;
+    const int64_t per_block = (int64_t)kThreads * kUnroll;
+    const int64_t blocks = (nvec + per_block - 1) / per_block;
+    if (blocks > 0x7fffffffLL) return KR_ERR_BAD_DIM;
+    const dim3 grid((unsigned)blocks);
+    const hipStream_t s = (hipStream_t)stream;
+    const u32x4* sp = (const u32x4*)stack;
+    const u32x4* bp = (const u32x4*)bias;
+    u32x4* op = (u32x4*)out;
+    const int64_t ssv = slice_stride / 8;
+    const uint32_t d_vec = mode == kVectorBias ? (uint32_t)(D / 8) : 1u;
+    hipError_t e;
+    switch (W) {
+        case 2: e = launch_reduce1<2>(mode, bias_first != 0, grid, s, sp, W, ssv, nvec, bp, d_vec, op); break;
+        case 4: e = launch_reduce1<4>(mode, bias_first != 0, grid, s, sp, W, ssv, nvec, bp, d_vec, op); break;
+        case 8: e = launch_reduce1<8>(mode, bias_first != 0, grid, s, sp, W, ssv, nvec, bp, d_vec, op); break;
+        default: e = launch_reduce1<0>(mode, bias_first != 0, grid, s, sp, W, ssv, nvec, bp, d_vec, op); break;
+    }
+    return (int)e;
+}
+
+extern "C" int64_t kr_striped_share_numel(int64_t numel, int W, int64_t stripe_block, int rank) {
+    if (W < 1 || W > KR_MAX_WORLD) return KR_ERR_WORLD_SIZE;
+    if (numel < 0) return KR_ERR_BAD_DIM;
+    if (numel % 8 != 0) return KR_ERR_NUMEL_MOD8;
+    if (stripe_block <= 0 || stripe_block % 8 != 0 || rank < 0 || rank >= W) return KR_ERR_STRIPE;
+    const int64_t stripe = stripe_block * W;
+    const int64_t full = numel / stripe;
+    const int64_t rem = numel - full * stripe;
+    int64_t tail = rem - (int64_t)rank * stripe_block;
+    if (tail < 0) tail = 0;
+    if (tail > stripe_block) tail = stripe_block;
+    return full * stripe_block + tail;
+}
+
+extern "C" int kr_reduce_striped_bf16(const void* stack, int W, int64_t slice_stride, int64_t numel,
+                                      const void* bias, int64_t stripe_block, int rank, void* out,
+                                      void* stream) {
+    const int64_t share = kr_striped_share_numel(numel, W, stripe_block, rank);
+    if (share < 0) return (int)share;
+    if (share == 0) return KR_OK;
+    int rc = check_reduce_common(stack, W, slice_stride, numel, out);
+    if (rc != KR_OK) return rc;
+    if (bias != nullptr && !aligned16(bias)) return KR_ERR_ALIGNMENT;
+    const int64_t nvec = share / 8;
+    const int64_t blocks = (nvec + kThreads - 1) / kThreads;
+    if (blocks > 0x7fffffffLL || stripe_block / 8 > 0xffffffffLL) return KR_ERR_BAD_DIM;
+    hipLaunchKernelGGL(reduce_striped_kernel, dim3((unsigned)blocks), dim3(kThreads), 0, (hipStream_t)stream,
+                       (const u32x4*)stack, W, slice_stride / 8, nvec, (const u32x4*)bias,
+                       (uint32_t)(stripe_block / 8), rank, (u32x4*)out);
+    return (int)hipGetLastError();
+}
+
+extern "C" int kr_reduce_rotated_bf16(const void* in, int W, int64_t rows, int64_t N, int rank, int acc_bf16,
+                                      void* out, void* stream) {
+    if (W < 1 || W > KR_MAX_WORLD) return KR_ERR_WORLD_SIZE;
+    if (rows < 0 || N < 0) return KR_ERR_BAD_DIM;
+    if (rank < 0 || rank >= W) return KR_ERR_STRIPE;
+    const int64_t band = rows * N;
+    if (band % 8 != 0) return KR_ERR_NUMEL_MOD8;
+    if (band == 0) return KR_OK;
+    if (in == nullptr || out == nullptr) return KR_ERR_NULL_POINTER;
+    if (!aligned16(in) || !aligned16(out)) return KR_ERR_ALIGNMENT;
+    const int64_t band_v = band / 8;
+    const int64_t blocks = (band_v + kThreads - 1) / kThreads;
+    if (blocks > 0x7fffffffLL) return KR_ERR_BAD_DIM;
+    if (acc_bf16)
+        hipLaunchKernelGGL((reduce_rotated_kernel<true>), dim3((unsigned)blocks), dim3(kThreads), 0,
+                           (hipStream_t)stream, (const u32x4*)in, W, band_v, rank, (u32x4*)out);
+    else
+        hipLaunchKernelGGL((reduce_rotated_kernel<false>), dim3((unsigned)blocks), dim3(kThreads), 0,
+                           (hipStream_t)stream, (const u32x4*)in, W, band_v, rank, (u32x4*)out);
+    return (int)hipGetLastError();
+}

@@ -1,0 +1,210 @@
+// Row kernels: W-way reduce + bias + RMSNorm in one pass, and stand-alone RMSNorm.
+//
+// One workgroup owns one row.  The reduced row lives in fp32 registers (VPT
+// 128-bit vectors per thread), so every input byte is read exactly once:
+// W*D*2 B of slices (+ D*2 bias + D*2 weight) in, D*2 B out per row.  The sum
+// of squares is reduced inside each wavefront with DPP lane permutes, then
+// across the wavefronts of the workgroup through a few words of LDS that every
+// thread re-reads in the same order, so all threads hold the same rstd.
+#include "common.h"
+
+namespace kr {
+
+enum RowBias { kRowNoBias = 0, kRowFullBias = 1, kRowVecBias = 2 };
+
+constexpr int kMaxVpt = 8;       // vectors per thread  -> D <= 1024 * 8 * 8
+constexpr int kMaxThreads = 1024;
+
+template <int VPT, int WT, int BIAS>
+__global__ __launch_bounds__(kMaxThreads) void reduce_rmsnorm_kernel(
+    const u32x4* __restrict__ stack, int w_rt, int64_t slice_stride_v, int d_vec,
+    const u32x4* __restrict__ bias, const u32x4* __restrict__ wgt, float eps, float inv_d,
+    u32x4* __restrict__ y) {
+    __shared__ float wave_part[kMaxThreads / kWave];
+    const int W = WT > 0 ? WT : w_rt;
+    const int tid = threadIdx.x;
+    const int nthr = blockDim.x;
+    const int64_t row_v = (int64_t)blockIdx.x * d_vec;
+
+    float s[VPT][8];
+    u32x4 wv[VPT];
+
+    // issue the weight loads early; they are shared by all rows and stay in L2
+#pragma unroll
+    for (int v = 0; v < VPT; ++v) {
+        const int c = tid + v * nthr;
+        wv[v] = c < d_vec ? wgt[c] : u32x4{0, 0, 0, 0};
+    }
+
+#pragma unroll
+    for (int v = 0; v < VPT; ++v) {
+        const int c = tid + v * nthr;
+        if (BIAS == kRowNoBias || c >= d_vec) {
+            zero8(s[v]);
+        } else if (BIAS == kRowFullBias) {
+            unpack8(ld_stream(bias + row_v + c), s[v]);
+        } else {
+            unpack8(bias[c], s[v]);
+        }
+    }
+
+    if constexpr (WT > 0 && WT * VPT <= 16) {
+        // all W*VPT loads of the thread in flight before the first add
+        u32x4 x[WT][VPT];
+#pragma unroll
+        for (int r = 0; r < WT; ++r)
+#pragma unroll
+            for (int v = 0; v < VPT; ++v) {
+                const int c = tid + v * nthr;
+                x[r][v] = c < d_vec ? ld_stream(stack + r * slice_stride_v + row_v + c) : u32x4{0, 0, 0, 0};
+            }
+#pragma unroll
+        for (int r = 0; r < WT; ++r)
+#pragma unroll
+            for (int v = 0; v < VPT; ++v) add8(x[r][v], s[v]);
+    } else {
+        // long rows: one slice at a time keeps the register count bounded
+        for (int r = 0; r < W; ++r) {
+            u32x4 x[VPT];
+#pragma unroll
+            for (int v = 0; v < VPT; ++v) {
+                const int c = tid + v * nthr;
+                x[v] = c < d_vec ? ld_stream(stack + r * slice_stride_v + row_v + c) : u32x4{0, 0, 0, 0};
+            }
+#pragma unroll
+            for (int v = 0; v < VPT; ++v) add8(x[v], s[v]);
+        }
+    }
+
+    float ss = 0.0f;
+#pragma unroll
+    for (int v = 0; v < VPT; ++v)
+#pragma unroll
+        for (int j = 0; j < 8; ++j) ss += s[v][j] * s[v][j];
+
+    ss = wave_sum(ss);
+    const int nwaves = nthr / kWave;
+    float total = ss;
+    if (nwaves > 1) {
+        if ((tid & (kWave - 1)) == 0) wave_part[tid / kWave] = ss;
+        __syncthreads();
+        total = 0.0f;
+        for (int i = 0; i < nwaves; ++i) total += wave_part[i];
+    }
+    const float rstd = __builtin_amdgcn_rsqf(total * inv_d + eps);
+
+#pragma unroll
+    for (int v = 0; v < VPT; ++v) {
+        const int c = tid + v * nthr;
+        if (c < d_vec) {
+            float wf[8], o[8];
+            unpack8(wv[v], wf);
+#pragma unroll
+            for (int j = 0; j < 8; ++j) o[j] = (s[v][j] * rstd) * wf[j];
+            st_stream(y + row_v + c, pack8(o));
+        }
+    }
+}
+
+template <int VPT, int WT>
+static hipError_t launch_row2(int mode, dim3 grid, dim3 block, hipStream_t st, const u32x4* stack, int W,
+                              int64_t ssv, int d_vec, const u32x4* bias, const u32x4* wgt, float eps,
+                              float inv_d, u32x4* y) {
+    switch (mode) {
+        case kRowNoBias:
+            hipLaunchKernelGGL((reduce_rmsnorm_kernel<VPT, WT, kRowNoBias>), grid, block, 0, st, stack, W, ssv,
+                               d_vec, bias, wgt, eps, inv_d, y);
+            break;
+        case kRowFullBias:
+            hipLaunchKernelGGL((reduce_rmsnorm_kernel<VPT, WT, kRowFullBias>), grid, block, 0, st, stack, W, ssv,
+                               d_vec, bias, wgt, eps, inv_d, y);
+            break;
+        default:
+            hipLaunchKernelGGL((reduce_rmsnorm_kernel<VPT, WT, kRowVecBias>), grid, block, 0, st, stack, W, ssv,
+                               d_vec, bias, wgt, eps, inv_d, y);
+            break;
+    }
+    return hipGetLastError();
+}
+
+template <int VPT>
+static hipError_t launch_row1(int W, int mode, dim3 grid, dim3 block, hipStream_t st, const u32x4* stack,
+                              int64_t ssv, int d_vec, const u32x4* bias, const u32x4* wgt, float eps,
+                              float inv_d, u32x4* y) {
+    switch (W) {
+        case 1: return launch_row2<VPT, 1>(mode, grid, block, st, stack, W, ssv, d_vec, bias, wgt, eps, inv_d, y);
+        case 2: return launch_row2<VPT, 2>(mode, grid, block, st, stack, W, ssv, d_vec, bias, wgt, eps, inv_d, y);
+        case 4: return launch_row2<VPT, 4>(mode, grid, block, st, stack, W, ssv, d_vec, bias, wgt, eps, inv_d, y);
+        case 8: return launch_row2<VPT, 8>(mode, grid, block, st, stack, W, ssv, d_vec, bias, wgt, eps, inv_d, y);
+        default: return launch_row2<VPT, 0>(mode, grid, block, st, stack, W, ssv, d_vec, bias, wgt, eps, inv_d, y);
+    }
+}
+
+// Threads per row: enough 64-lane wavefronts to give every thread at most
+// `vpt` vectors, capped at 1024 threads.
+static void row_geometry(int d_vec, int* threads, int* vpt) {
+    int v = 1;
+    while ((int64_t)v * kMaxThreads < d_vec) v *= 2;           // 1,2,4,8
+    // prefer 2 vectors per thread once a row spans more than 256 vectors: fewer
+    // wavefronts to synchronise, same bytes in flight per CU
+    if (v == 1 && d_vec > 256) v = 2;
+    int t = (d_vec + v - 1) / v;
+    t = (t + kWave - 1) / kWave * kWave;
+    *threads = t;
+    *vpt = v;
+}
+
+static int launch_rows(const void* stack, int W, int64_t slice_stride, int64_t rows, int64_t D, const void* bias,
+                       int mode, const void* w, float eps, void* y, void* stream) {
+    int threads, vpt;
+    const int d_vec = (int)(D / 8);
+    row_geometry(d_vec, &threads, &vpt);
+    const dim3 grid((unsigned)rows), block((unsigned)threads);
+    const hipStream_t st = (hipStream_t)stream;
+    const u32x4* sp = (const u32x4*)stack;
+    const u32x4* bp = (const u32x4*)bias;
+    const u32x4* wp = (const u32x4*)w;
+    u32x4* yp = (u32x4*)y;
+    const int64_t ssv = slice_stride / 8;
+    const float inv_d = 1.0f / (float)D;
+    hipError_t e;
+    switch (vpt) {
+        case 1: e = launch_row1<1>(W, mode, grid, block, st, sp, ssv, d_vec, bp, wp, eps, inv_d, yp); break;
+        case 2: e = launch_row1<2>(W, mode, grid, block, st, sp, ssv, d_vec, bp, wp, eps, inv_d, yp); break;
+        case 4: e = launch_row1<4>(W, mode, grid, block, st, sp, ssv, d_vec, bp, wp, eps, inv_d, yp); break;
+        default: e = launch_row1<8>(W, mode, grid, block, st, sp, ssv, d_vec, bp, wp, eps, inv_d, yp); break;
+    }
+    return (int)e;
+}
+
+}  // namespace kr
+
+using namespace kr;
+
+extern "C" int kr_reduce_rmsnorm_bf16(const void* stack, int W, int64_t slice_stride, int64_t rows, int64_t D,
+                                      const void* bias, int bias_is_vector, const void* w, float eps, void* y,
+                                      void* stream) {
+    if (W < 1 || W > KR_MAX_WORLD) return KR_ERR_WORLD_SIZE;
+    if (rows < 0 || D <= 0 || slice_stride < 0) return KR_ERR_BAD_DIM;
+    if (D % 8 != 0) return KR_ERR_NUMEL_MOD8;
+    if (D > KR_MAX_ROW) return KR_ERR_ROW_TOO_LONG;
+    if (rows > 0x7fffffffLL) return KR_ERR_BAD_DIM;
+    if (rows == 0) return KR_OK;
+    if (stack == nullptr || w == nullptr || y == nullptr) return KR_ERR_NULL_POINTER;
+    if (!aligned16(stack) || !aligned16(w) || !aligned16(y) || slice_stride % 8 != 0) return KR_ERR_ALIGNMENT;
+    if (bias != nullptr && !aligned16(bias)) return KR_ERR_ALIGNMENT;
+    const int mode = bias == nullptr ? kRowNoBias : (bias_is_vector ? kRowVecBias : kRowFullBias);
+    return launch_rows(stack, W, slice_stride, rows, D, bias, mode, w, eps, y, stream);
+}
+
+extern "C" int kr_rmsnorm_bf16(const void* x, const void* w, float eps, int64_t rows, int64_t D, void* y,
+                               void* stream) {
+    if (rows < 0 || D <= 0) return KR_ERR_BAD_DIM;
+    if (D % 8 != 0) return KR_ERR_NUMEL_MOD8;
+    if (D > KR_MAX_ROW) return KR_ERR_ROW_TOO_LONG;
+    if (rows > 0x7fffffffLL) return KR_ERR_BAD_DIM;
+    if (rows == 0) return KR_OK;
+    if (x == nullptr || w == nullptr || y == nullptr) return KR_ERR_NULL_POINTER;
+    if (!aligned16(x) || !aligned16(w) || !aligned16(y)) return KR_ERR_ALIGNMENT;
+    return launch_rows(x, 1, 0, rows, D, nullptr, kRowNoBias, w, eps, y, stream);
+}

@@ -1,0 +1,23 @@
+// Version and error-text entry points of the C ABI.
+#include "common.h"
+
+extern "C" int kr_version(void) { return 100; }  // 0.1.0
+
+extern "C" const char* kr_strerror(int code) {
+    switch (code) {
+        case KR_OK: return "success";
+        case KR_ERR_NULL_POINTER: return "a required pointer is NULL";
+        case KR_ERR_ALIGNMENT: return "pointer or stride is not 16-byte (128-bit) aligned";
+        case KR_ERR_NUMEL_MOD8: return "the number of elements must be 128-bit aligned (a multiple of 8 bf16)";
+        case KR_ERR_BAD_DIM: return "negative, zero or inconsistent dimension";
+        case KR_ERR_WORLD_SIZE: return "world size outside 1..16";
+        case KR_ERR_BIAS_SHAPE: return "bias must have the shape of the input or be a vector of the last dimension";
+        case KR_ERR_ROW_TOO_LONG: return "row length above 65536 is not supported by the row-resident kernels";
+        case KR_ERR_BAND: return "row band outside [0, M)";
+        case KR_ERR_LAYOUT: return "operand strides not supported (A must be k-contiguous; B row-major or transposed-contiguous)";
+        case KR_ERR_STRIPE: return "stripe block must be a positive multiple of 8 and 0 <= rank < W";
+        default: break;
+    }
+    if (code > 0) return hipGetErrorString((hipError_t)code);
+    return "unknown kraken_amd error code";
+}

@@ -1,0 +1,71 @@
+"""Shared host logic of the GEMM + reduce wrappers."""
+from __future__ import annotations
+
+import torch
+
+from .. import _lib
+
+
+def split_fp32(a: torch.Tensor, b: torch.Tensor) -> tuple[torch.Tensor, torch.Tensor]:
+    """fp32 operands for the bf16 matrix cores: a = a_hi + a_lo, b = b_hi + b_lo.
+
+    ``[a_hi | a_hi | a_lo] @ [b_hi ; b_lo ; b_hi]`` (one GEMM with 3K inner
+    length, fp32 accumulate) equals ``a@b`` up to the dropped ``a_lo@b_lo``
+    term, i.e. about 16 mantissa bits — tighter than the TF32 ``tl.dot`` the
+    reference runs fp32 inputs through (``gemm_one_shot_all_reduce_fused.py:56-64``).
+    """
+    a_hi = a.to(torch.bfloat16)
+    a_lo = (a - a_hi.float()).to(torch.bfloat16)
+    b_hi = b.to(torch.bfloat16)
+    b_lo = (b - b_hi.float()).to(torch.bfloat16)
+    return torch.cat([a_hi, a_hi, a_lo], dim=1), torch.cat([b_hi, b_lo, b_hi], dim=0)
+
+
+def prepare_operands(a: torch.Tensor, b: torch.Tensor) -> tuple[torch.Tensor, torch.Tensor]:
+    """Return bf16 operands in a layout the kernel reads directly.
+
+    A must be k-contiguous; B either row-major or transposed-contiguous.  Other
+    stridings (the reference accepts any 2-D strides) are made contiguous.
+    K and N are padded to multiples of 8 with zeros when necessary.
+    """
+    assert a.dim() == 2 and b.dim() == 2
+    assert a.shape[1] == b.shape[0], "Inner dimensions must match for matrix multiplication"
+    assert a.dtype == b.dtype, "Input tensors must have the same dtype"
+    assert a.dtype in (torch.bfloat16, torch.float32), "bfloat16 (or float32) operands expected"
+    if a.dtype == torch.float32:
+        a, b = split_fp32(a, b)
+    K = a.shape[1]
+    if K % 8 != 0:
+        pad = 8 - K % 8
+        a = torch.nn.functional.pad(a, (0, pad))
+        b = torch.nn.functional.pad(b, (0, 0, 0, pad))
+    if a.stride(1) != 1 or a.stride(0) % 8 != 0 or a.data_ptr() % 16 != 0:
+        a = a.contiguous()
+    b_ok = (b.stride(1) == 1 and b.stride(0) % 8 == 0) or (b.stride(0) == 1 and b.stride(1) % 8 == 0)
+    if not b_ok or b.data_ptr() % 16 != 0:
+        b = b.contiguous()
+    return a, b
+
+
+def launch(name, a, b, M, N, peers, n_peers, peers_stride, bias, band_row0, band_rows, c_full, out, pivot):
+    dev = _lib.require_device(a, b, peers, bias, c_full, out)
+    rc = _lib.load().kr_gemm_reduce_bf16(
+        a.data_ptr(), a.stride(0), a.stride(1), b.data_ptr(), b.stride(0), b.stride(1),
+        M, N, a.shape[1], _lib.ptr(peers), n_peers, peers_stride, _lib.ptr(bias),
+        band_row0, band_rows, _lib.ptr(c_full), _lib.ptr(out),
+        int(out is not None and out.dtype == torch.float32), pivot, _lib.current_stream(dev),
+    )
+    _lib.check(rc, name)
+
+
+def check_peers(peers: torch.Tensor | None, rows: int, N: int) -> tuple[int, int]:
+    """Validate pre-staged partials ``[P, rows, N]``; return (P, stride)."""
+    if peers is None:
+        return 0, 0
+    assert peers.dtype == torch.bfloat16, "pre-staged partials must be bfloat16"
+    assert peers.dim() == 3 and tuple(peers.shape[1:]) == (rows, N), (
+        f"peers must have shape [W-1, {rows}, {N}], got {tuple(peers.shape)}"
+    )
+    assert peers[0].is_contiguous()
+    P = peers.shape[0]
+    return P, (peers.stride(0) if P > 1 else rows * N)

@@ -1,0 +1,172 @@
+"""Host side of the C ABI, exercised without a GPU: the library loads, exports every symbol
+include/kraken_amd.h declares, and rejects bad arguments before any launch.  The Python
+wrappers raise like the reference's asserts and refuse host tensors (no CPU fallback)."""
+import ctypes
+import re
+from pathlib import Path
+
+import pytest
+import torch
+
+import kraken_amd
+from kraken_amd import _lib, comm, fused
+
+ROOT = Path(__file__).resolve().parent.parent
+BF16 = torch.bfloat16
+FAKE = 0x10000  # aligned, non-null; never dereferenced because validation fails first
+
+
+@pytest.fixture(scope="module")
+def lib():
+    return _lib.load()
+
+
+def test_library_exports_every_declared_symbol(lib):
+    header = (ROOT / "include" / "kraken_amd.h").read_text()
+    declared = set(re.findall(r"\b(kr_[a-z0-9_]+)\s*\(", header))
+    assert declared, "no declarations found"
+    assert declared == set(_lib.EXPORTS)
+    raw = ctypes.CDLL(str(_lib.LIB_PATH))
+    for name in declared:
+        assert hasattr(raw, name), f"{name} not exported"
+    assert lib.kr_version() >= 100
+
+
+def test_strerror_known_and_unknown(lib):
+    assert "128-bit" in _lib.strerror(_lib.KR_ERR_NUMEL_MOD8)
+    assert _lib.strerror(0) == "success"
+    assert "unknown" in _lib.strerror(-999)
+
+
+def test_reduce_argument_errors(lib):
+    f = lib.kr_reduce_bf16
+    assert f(FAKE, 8, 64, 12, None, 0, 0, 1, FAKE, None) == _lib.KR_ERR_NUMEL_MOD8
+    assert f(FAKE, 0, 64, 16, None, 0, 0, 1, FAKE, None) == _lib.KR_ERR_WORLD_SIZE
+    assert f(FAKE, 17, 64, 16, None, 0, 0, 1, FAKE, None) == _lib.KR_ERR_WORLD_SIZE
+    assert f(None, 8, 64, 16, None, 0, 0, 1, FAKE, None) == _lib.KR_ERR_NULL_POINTER
+    assert f(FAKE, 8, 64, 16, None, 0, 0, 1, None, None) == _lib.KR_ERR_NULL_POINTER
+    assert f(FAKE + 2, 8, 64, 16, None, 0, 0, 1, FAKE, None) == _lib.KR_ERR_ALIGNMENT
+    assert f(FAKE, 8, 60, 16, None, 0, 0, 1, FAKE, None) == _lib.KR_ERR_ALIGNMENT
+    assert f(FAKE, 8, 64, -8, None, 0, 0, 1, FAKE, None) == _lib.KR_ERR_BAD_DIM
+    assert f(FAKE, 8, 64, 64, FAKE, 24, 16, 1, FAKE, None) == _lib.KR_ERR_BIAS_SHAPE
+    assert f(FAKE, 8, 64, 64, FAKE + 4, 64, 16, 1, FAKE, None) == _lib.KR_ERR_ALIGNMENT
+    # empty input: nothing to do, nothing launched
+    assert f(None, 8, 0, 0, None, 0, 0, 1, None, None) == 0
+
+
+def test_rmsnorm_argument_errors(lib):
+    f = lib.kr_reduce_rmsnorm_bf16
+    assert f(FAKE, 8, 4096, 1, 4100, None, 0, FAKE, 1e-5, FAKE, None) == _lib.KR_ERR_NUMEL_MOD8
+    assert f(FAKE, 8, 1 << 20, 1, 65536 + 8, None, 0, FAKE, 1e-5, FAKE, None) == _lib.KR_ERR_ROW_TOO_LONG
+    assert f(FAKE, 8, 4096, 1, 4096, None, 0, None, 1e-5, FAKE, None) == _lib.KR_ERR_NULL_POINTER
+    assert f(FAKE, 99, 4096, 1, 4096, None, 0, FAKE, 1e-5, FAKE, None) == _lib.KR_ERR_WORLD_SIZE
+    assert f(FAKE, 8, 4096, 0, 4096, None, 0, FAKE, 1e-5, FAKE, None) == 0
+    g = lib.kr_rmsnorm_bf16
+    assert g(FAKE, FAKE, 1e-5, 4, 0, FAKE, None) == _lib.KR_ERR_BAD_DIM
+    assert g(FAKE, FAKE + 8, 1e-5, 4, 64, FAKE, None) == _lib.KR_ERR_ALIGNMENT
+
+
+def test_gemm_argument_errors(lib):
+    f = lib.kr_gemm_reduce_bf16
+
+    def call(**kw):
+        a = dict(A=FAKE, lda_m=64, lda_k=1, B=FAKE, ldb_k=64, ldb_n=1, M=64, N=64, K=64, peers=None,
+                 n_peers=0, pstride=0, bias=None, band0=0, band=64, c_full=None, out=FAKE, f32=0, pivot=0)
+        a.update(kw)
+        return f(a["A"], a["lda_m"], a["lda_k"], a["B"], a["ldb_k"], a["ldb_n"], a["M"], a["N"], a["K"],
+                 a["peers"], a["n_peers"], a["pstride"], a["bias"], a["band0"], a["band"], a["c_full"],
+                 a["out"], a["f32"], a["pivot"], None)
+
+    assert call(K=60) == _lib.KR_ERR_NUMEL_MOD8
+    assert call(N=60) == _lib.KR_ERR_NUMEL_MOD8
+    assert call(lda_k=2) == _lib.KR_ERR_LAYOUT
+    assert call(ldb_k=3, ldb_n=5) == _lib.KR_ERR_LAYOUT
+    assert call(band0=32, band=64) == _lib.KR_ERR_BAND
+    assert call(A=None) == _lib.KR_ERR_NULL_POINTER
+    assert call(out=None) == _lib.KR_ERR_NULL_POINTER
+    assert call(n_peers=3, peers=None) == _lib.KR_ERR_NULL_POINTER
+    assert call(n_peers=3, peers=FAKE, pstride=64) == _lib.KR_ERR_BAD_DIM
+    assert call(lda_m=68) == _lib.KR_ERR_ALIGNMENT
+    assert call(M=-1) == _lib.KR_ERR_BAD_DIM
+    assert call(M=0, band=0) == 0
+
+
+def test_striped_share_numel(lib):
+    f = lib.kr_striped_share_numel
+    numel, W, block = 8 * 37, 4, 16
+    shares = [f(numel, W, block, r) for r in range(W)]
+    assert sum(shares) == numel
+    from oracle import oracle as orc
+    assert shares == [orc.striped_indices(numel, W, block, r).numel() for r in range(W)]
+    assert f(numel, W, 12, 0) == _lib.KR_ERR_STRIPE
+    assert f(numel, W, 16, 4) == _lib.KR_ERR_STRIPE
+    assert f(numel + 4, W, 16, 0) == _lib.KR_ERR_NUMEL_MOD8
+
+
+def test_rotated_argument_errors(lib):
+    f = lib.kr_reduce_rotated_bf16
+    assert f(FAKE, 4, 3, 16, 4, 1, FAKE, None) == _lib.KR_ERR_STRIPE
+    assert f(FAKE, 4, 3, 12, 0, 1, FAKE, None) == _lib.KR_ERR_NUMEL_MOD8
+    assert f(None, 4, 3, 16, 0, 1, FAKE, None) == _lib.KR_ERR_NULL_POINTER
+
+
+def test_check_maps_codes_to_reference_exceptions():
+    with pytest.raises(AssertionError, match="128-bit"):
+        _lib.check(_lib.KR_ERR_NUMEL_MOD8, "x")
+    with pytest.raises(ValueError):
+        _lib.check(_lib.KR_ERR_LAYOUT, "x")
+    with pytest.raises(_lib.KrakenAmdError):
+        _lib.check(1, "x")
+    _lib.check(0, "x")
+
+
+def test_public_names_match_reference_layout():
+    # kraken/comm/__init__.py:12-17 (reduce entry points), kraken/fused/__init__.py:17-27
+    assert set(comm.__all__) == {"one_shot_all_reduce", "two_shot_all_reduce"}
+    assert set(fused.__all__) == {
+        "all_gather_matmul", "gemm_one_shot_all_reduce_fused", "gemm_reduce_scatter",
+        "gemm_reduce_scatter_ce_persistent", "one_shot_all_reduce_bias",
+        "one_shot_all_reduce_bias_rms_norm", "rms_norm", "two_shot_all_reduce_bias",
+        "two_shot_all_reduce_bias_rms_norm",
+    }
+    assert kraken_amd.__all__ == ["_lib", "_logging", "comm", "fused"]
+
+
+def test_wrappers_assert_like_the_reference_and_refuse_host_tensors():
+    s32 = torch.zeros(8, 4, 64, dtype=torch.float32)
+    with pytest.raises(AssertionError, match="bfloat16"):
+        comm.one_shot_all_reduce(s32)                       # one_shot_all_reduce.py:79
+    with pytest.raises(AssertionError, match="128-bit"):
+        comm.one_shot_all_reduce(torch.zeros(8, 3, 4, dtype=BF16))   # :80
+    with pytest.raises(AssertionError):
+        comm.two_shot_all_reduce(torch.zeros(3, 8, 64, dtype=BF16), BLOCK_SIZE=2048)  # BLOCK % W
+    s = torch.zeros(8, 4, 64, dtype=BF16)
+    with pytest.raises(RuntimeError, match="no CPU fallback"):
+        comm.one_shot_all_reduce(s)
+    y = torch.empty(4, 64, dtype=BF16)
+    w = torch.ones(64, dtype=BF16)
+    with pytest.raises(AssertionError):
+        fused.one_shot_all_reduce_bias_rms_norm(s, None, None, torch.ones(32, dtype=BF16), y)  # w.shape == (D,)
+    with pytest.raises(AssertionError):
+        fused.two_shot_all_reduce_bias_rms_norm(torch.zeros(8, 1, 72, dtype=BF16), None, None,
+                                                torch.ones(72, dtype=BF16), torch.empty(1, 72, dtype=BF16))
+    with pytest.raises(RuntimeError, match="no CPU fallback"):
+        fused.one_shot_all_reduce_bias_rms_norm(s, None, None, w, y)
+    with pytest.raises(RuntimeError, match="no CPU fallback"):
+        fused.rms_norm(torch.zeros(4, 64, dtype=BF16), w)
+    a, b = torch.zeros(64, 32, dtype=BF16), torch.zeros(32, 64, dtype=BF16)
+    with pytest.raises(AssertionError, match="Inner dimensions"):
+        fused.gemm_one_shot_all_reduce_fused(a, torch.zeros(16, 64, dtype=BF16))
+    with pytest.raises(AssertionError, match="divisible by world_size"):
+        fused.gemm_reduce_scatter(torch.zeros(66, 32, dtype=BF16), b, world_size=4)
+    with pytest.raises(ValueError, match="b.T must be contiguous"):
+        fused.all_gather_matmul(torch.zeros(4, 16, 32, dtype=BF16), b)   # all_gather_matmul.py:158-160
+    with pytest.raises(RuntimeError, match="no CPU fallback"):
+        fused.gemm_one_shot_all_reduce_fused(a, b)
+
+
+def test_missing_library_fails_loudly(monkeypatch, tmp_path):
+    monkeypatch.setattr(_lib, "_lib", None)
+    monkeypatch.setattr(_lib, "LIB_PATH", tmp_path / "libkraken_amd.so")
+    with pytest.raises(RuntimeError, match="kraken_amd.build"):
+        _lib.load()

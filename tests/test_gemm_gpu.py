@@ -1,0 +1,187 @@
+"""GPU parity of the bf16 MFMA GEMM with fused reduce(+bias) epilogue against the CPU oracle.
+Gate: rtol = atol = 2e-2 for bf16 outputs vs the fp32-accumulated oracle."""
+import os
+
+import pytest
+import torch
+
+from kraken_amd import fused
+from oracle import oracle as orc
+
+pytestmark = pytest.mark.gpu
+BF16 = torch.bfloat16
+TOL = dict(rtol=2e-2, atol=2e-2)
+
+
+@pytest.fixture(params=["128", "256"])
+def tile(request, monkeypatch):
+    monkeypatch.setenv("KRAKEN_AMD_GEMM_TILE", request.param)
+    return request.param
+
+
+def mk(M, N, K, P, b_t=False, seed=0):
+    a = orc.randn_bf16((M, K), 42 + seed)
+    if b_t:
+        b = orc.randn_bf16((N, K), 43 + seed, 0.05).T          # b.T contiguous
+    else:
+        b = orc.randn_bf16((K, N), 43 + seed, 0.05)
+    peers = torch.stack([orc.randn_bf16((M, N), 100 + j) for j in range(P)]) if P else None
+    return a, b, peers
+
+
+def test_rank_specific_known_answer(dev, tile):
+    # test/test_gemm_allreduce.py:92-117 (M=N=K=32, W=4): every element K*(1+2+3+4), at 1e-5
+    M = N = K = 32
+    a = torch.ones(M, K, dtype=BF16)
+    b = torch.ones(K, N, dtype=BF16)
+    peers = torch.stack([torch.full((M, N), float((r + 1) * K), dtype=BF16) for r in range(1, 4)])
+    out = fused.gemm_one_shot_all_reduce_fused(a.to(dev), b.to(dev), peers=peers.to(dev))
+    assert out.dtype == torch.float32 and out.shape == (M, N)
+    torch.testing.assert_close(out.cpu(), torch.full((M, N), float(K * 10)), rtol=1e-5, atol=1e-5)
+    # same with fp32 operands, as the reference test passes them
+    out32 = fused.gemm_one_shot_all_reduce_fused(a.float().to(dev), b.float().to(dev), peers=peers.to(dev))
+    torch.testing.assert_close(out32.cpu(), torch.full((M, N), float(K * 10)), rtol=1e-5, atol=1e-5)
+
+
+@pytest.mark.parametrize("shape", [(512, 256, 128), (256, 256, 256), (128, 128, 64), (384, 640, 192),
+                                   (100, 72, 40), (8, 8, 8), (1000, 264, 520)])
+@pytest.mark.parametrize("b_t", [False, True])
+def test_gemm_all_reduce_shapes(dev, tile, shape, b_t):
+    M, N, K = shape
+    a, b, peers = mk(M, N, K, 3, b_t)
+    bias = orc.randn_bf16((N,), 42, 0.02)
+    want = orc.gemm_all_reduce(a, b, peers, bias)
+    out = fused.gemm_one_shot_all_reduce_fused(a.to(dev), b.to(dev), peers=peers.to(dev), bias=bias.to(dev))
+    torch.testing.assert_close(out.cpu(), want, rtol=1e-3, atol=1e-3)      # fp32 out: tight
+    outb = fused.gemm_one_shot_all_reduce_fused(a.to(dev), b.to(dev), peers=peers.to(dev), bias=bias.to(dev),
+                                                out_dtype=BF16)
+    torch.testing.assert_close(outb.cpu(), want.to(BF16), **TOL)
+    plain = fused.gemm_one_shot_all_reduce_fused(a.to(dev), b.to(dev))
+    torch.testing.assert_close(plain.cpu(), orc.gemm_all_reduce(a, b), rtol=1e-3, atol=1e-3)
+
+
+def test_fp32_operands_reference_shapes(dev, tile):
+    # test/test_gemm_allreduce.py:51-89: fp32 N(0,1) operands, (512,256,128) and (256,256,256), tol 1e-1
+    for (M, N, K) in [(512, 256, 128), (256, 256, 256)]:
+        g = torch.Generator().manual_seed(42)
+        a = torch.randn(M, K, generator=g)
+        b = torch.randn(K, N, generator=g)
+        out = fused.gemm_one_shot_all_reduce_fused(a.to(dev), b.to(dev))
+        torch.testing.assert_close(out.cpu(), a @ b, rtol=1e-1, atol=1e-1)
+        torch.testing.assert_close(out.cpu(), a @ b, rtol=2e-3, atol=2e-3)   # the split keeps ~16 bits
+
+
+@pytest.mark.parametrize("rank", [0, 2, 3])
+@pytest.mark.parametrize("b_t", [False, True])
+def test_gemm_reduce_scatter(dev, tile, rank, b_t):
+    M, N, K, W = 512, 256, 128, 4        # test/test_gemm_reduce_scatter.py:61-74
+    a, b, _ = mk(M, N, K, 0, b_t)
+    peers = torch.stack([orc.randn_bf16((M // W, N), 100 + j) for j in range(W - 1)])
+    want, c_want = orc.gemm_reduce_scatter(a, b, peers, rank, W)
+    c_scratch = torch.full((M, N), float("nan"), dtype=BF16, device=dev)
+    out = fused.gemm_reduce_scatter(a.to(dev), b.to(dev), peers=peers.to(dev), rank=rank, c_scratch=c_scratch)
+    assert out.shape == (M // W, N) and out.dtype == BF16
+    torch.testing.assert_close(out.cpu(), want, **TOL)
+    rows = torch.ones(M, dtype=torch.bool)
+    rows[rank * M // W:(rank + 1) * M // W] = False
+    torch.testing.assert_close(c_scratch.cpu()[rows], c_want[rows], **TOL)
+    assert torch.isnan(c_scratch.cpu()[~rows].float()).all()    # own band never makes the round trip
+
+
+def test_gemm_reduce_scatter_rank_specific(dev, tile):
+    # test/test_gemm_reduce_scatter.py:76-91
+    M, N, K, W = 512, 256, 128, 4
+    for rank in range(W):
+        a = torch.full((M, K), float(rank + 1), dtype=BF16)
+        b = torch.ones(K, N, dtype=BF16)
+        others = [r for r in range(W) if r != rank]
+        peers = torch.stack([torch.full((M // W, N), float((r + 1) * K), dtype=BF16) for r in others])
+        out = fused.gemm_reduce_scatter(a.to(dev), b.to(dev), peers=peers.to(dev), rank=rank)
+        assert torch.equal(out.cpu().float(), torch.full((M // W, N), float(K * 10)))
+
+
+@pytest.mark.parametrize("rank", [0, 3])
+def test_all_gather_matmul(dev, tile, rank):
+    W, m, K, N = 4, 128, 256, 384
+    stack = orc.make_stack(W, (m, K))
+    bT = orc.randn_bf16((N, K), 43, 0.05)
+    sd = stack.to(dev)
+    progress = torch.zeros(W, dtype=torch.int32, device=dev)
+    ag, c = fused.all_gather_matmul(sd, bT.to(dev).T, progress=progress, rank=rank)
+    a_want, c_want = orc.all_gather_matmul(stack, bT.T)
+    assert torch.equal(ag.cpu(), a_want)                      # test/test_allgather_matmul.py:75: exact
+    assert ag.data_ptr() == sd.data_ptr()                     # zero-copy view
+    assert (progress != 0).all()                              # test/test_allgather.py:73
+    torch.testing.assert_close(c.cpu(), c_want, **TOL)
+    a_out = torch.empty(W * m, K, dtype=BF16, device=dev)
+    ag2, c2 = fused.all_gather_matmul(sd, bT.to(dev).T, a_out=a_out, rank=rank)
+    assert ag2 is a_out and torch.equal(a_out.cpu(), a_want) and torch.equal(c2, c)
+
+
+def test_ce_persistent_variant(dev, tile):
+    M, N, K, W = 512, 256, 128, 4
+    a, b, _ = mk(M, N, K, 0, True)
+    for rank in (0, 2):
+        peers = torch.stack([orc.randn_bf16((M // W, N), 100 + j) for j in range(W - 1)])
+        out = fused.gemm_reduce_scatter_ce_persistent(a.to(dev), b.to(dev), peers=peers.to(dev), rank=rank)
+        c = (a.float() @ b.float()).to(BF16)
+        bands = list(peers)
+        bands.insert(rank, c[rank * M // W:(rank + 1) * M // W])
+        want = orc.reduce_rotated(torch.cat(bands, 0), W, rank, acc_bf16=True)
+        torch.testing.assert_close(out.cpu(), want, **TOL)
+
+
+def _sampled_rows_check(got, rows, a, b, extra, tol=TOL):
+    want = a[rows].float() @ b.float()
+    if extra is not None:
+        want = want + extra
+    torch.testing.assert_close(got.cpu()[rows].float(), want.to(BF16).float(), **tol)
+
+
+def test_baseline_config4_full_size(dev, monkeypatch):
+    """A [8192,3584] @ B [3584,8192]; band of 1024 rows + 7 partials.  Oracle on sampled rows."""
+    monkeypatch.delenv("KRAKEN_AMD_GEMM_TILE", raising=False)
+    M, N, K, W, rank = 8192, 8192, 3584, 8, 3
+    a = orc.randn_bf16((M, K), 42)
+    b = orc.randn_bf16((K, N), 43, 0.02)
+    peers = torch.stack([orc.randn_bf16((M // W, N), 100 + j) for j in range(W - 1)])
+    c_scratch = torch.empty(M, N, dtype=BF16, device=dev)
+    out = fused.gemm_reduce_scatter(a.to(dev), b.to(dev), peers=peers.to(dev), rank=rank, c_scratch=c_scratch)
+    band = torch.arange(rank * 1024, (rank + 1) * 1024)
+    pick = band[torch.tensor([0, 1, 31, 32, 255, 256, 511, 777, 1023])]
+    want = a[pick].float() @ b.float() + peers[:, pick - rank * 1024].float().sum(0)
+    torch.testing.assert_close(out.cpu()[pick - rank * 1024].float(), want.to(BF16).float(), **TOL)
+    others = torch.tensor([0, 255, 256, 1023, 4096, 5000, 8191])
+    _sampled_rows_check(c_scratch, others, a, b, None)
+    # whole-matrix check against the device library GEMM in fp32
+    ref = (a.to(dev).float() @ b.to(dev).float())
+    ref_band = ref[band.to(dev)] + peers.to(dev).float().sum(0)
+    torch.testing.assert_close(out.float(), ref_band.to(BF16).float(), **TOL)
+
+
+def test_baseline_config5_full_size(dev, monkeypatch):
+    monkeypatch.delenv("KRAKEN_AMD_GEMM_TILE", raising=False)
+    # fused all-reduce: A [4096,1024] @ B [1024,8192] + 7 partials + bias
+    M, N, K, P = 4096, 8192, 1024, 7
+    a = orc.randn_bf16((M, K), 42)
+    b = orc.randn_bf16((K, N), 43, 0.02)
+    peers = torch.stack([orc.randn_bf16((M, N), 100 + j) for j in range(P)])
+    bias = orc.randn_bf16((N,), 42, 0.02)
+    out = fused.gemm_one_shot_all_reduce_fused(a.to(dev), b.to(dev), peers=peers.to(dev), bias=bias.to(dev),
+                                               out_dtype=BF16)
+    pick = torch.tensor([0, 63, 64, 127, 128, 2047, 4095])
+    want = a[pick].float() @ b.float() + peers[:, pick].float().sum(0) + bias.float()
+    torch.testing.assert_close(out.cpu()[pick].float(), want.to(BF16).float(), **TOL)
+    ref = a.to(dev).float() @ b.to(dev).float() + peers.to(dev).float().sum(0) + bias.to(dev).float()
+    torch.testing.assert_close(out.float(), ref.to(BF16).float(), **TOL)
+    del peers, out, ref
+    # all-gather matmul: A stack [8,1024,8192] @ B [8192,3584] (B.T contiguous)
+    W, m, K2, N2 = 8, 1024, 8192, 3584
+    stack = orc.make_stack(W, (m, K2), seed0=42)
+    bT = orc.randn_bf16((N2, K2), 43, 0.02)
+    ag, c = fused.all_gather_matmul(stack.to(dev), bT.to(dev).T, rank=5)
+    assert torch.equal(ag.cpu(), stack.reshape(W * m, K2))
+    rows = torch.tensor([0, 1023, 1024, 5 * 1024, 5 * 1024 + 17, 8191])
+    _sampled_rows_check(c, rows, stack.reshape(W * m, K2), bT.T, None)
+    ref = stack.to(dev).reshape(W * m, K2).float() @ bT.to(dev).T.float()
+    torch.testing.assert_close(c.float(), ref.to(BF16).float(), **TOL)

@@ -1,0 +1,107 @@
+"""GPU parity of reduce+bias+RMSNorm and stand-alone RMSNorm against the CPU oracle.
+Gate: rtol = atol = 2e-2 (bf16 output vs fp32-accumulated reference); additionally the
+results must be within one bf16 ulp of the oracle (only the fp32 order of the sum of
+squares and the rsqrt approximation differ)."""
+import pytest
+import torch
+
+from kraken_amd import fused
+from oracle import oracle as orc
+
+pytestmark = pytest.mark.gpu
+BF16 = torch.bfloat16
+TOL = dict(rtol=2e-2, atol=2e-2)
+
+
+def assert_one_ulp(got, want):
+    g, w = got.cpu().float(), want.float()
+    d = (g - w).abs()
+    assert (d <= w.abs() * 2.0 ** -7 + 1e-30).all(), float(d.max())
+    assert (d == 0).float().mean() > 0.97
+
+
+@pytest.mark.parametrize("D", [8, 64, 320, 2048, 4096, 5120, 8192, 16384, 65536])
+@pytest.mark.parametrize("rows", [1, 5])
+def test_rms_norm_row_lengths(dev, D, rows):
+    x = orc.randn_bf16((rows, D), 3)
+    w = orc.randn_bf16((D,), 4)
+    y = fused.rms_norm(x.to(dev), w.to(dev), 1e-5)
+    want = orc.rms_norm(x, w, 1e-5)
+    torch.testing.assert_close(y.cpu(), want, **TOL)
+    assert_one_ulp(y, want)
+
+
+def test_rms_norm_closed_forms(dev):
+    D = 1024
+    w = orc.randn_bf16((D,), 6, 0.02, 1.0)
+    x = torch.full((3, D), 3.0, dtype=BF16)
+    y = fused.rms_norm(x.to(dev), w.to(dev), 1e-5).cpu()
+    want = (w.float() * (3.0 / (9.0 + 1e-5) ** 0.5)).to(BF16)
+    assert_one_ulp(y[1], want)
+    z = fused.rms_norm(torch.zeros(3, D, dtype=BF16, device=dev), w.to(dev)).cpu()
+    assert torch.equal(z, torch.zeros(3, D, dtype=BF16))
+    yy = fused.rms_norm(orc.randn_bf16((4, D), 8).to(dev), torch.ones(D, dtype=BF16, device=dev)).float()
+    torch.testing.assert_close((yy * yy).mean(-1).cpu(), torch.ones(4), rtol=1e-2, atol=1e-2)
+
+
+@pytest.mark.parametrize("b", [1, 2, 4, 8, 16, 32, 64])
+def test_reference_test_shapes(dev, b):
+    # test/test_allreduce_bias_rms_norm.py:56-86: x [b,5120] seed 42+rank+b, bias [b,5120] and
+    # w [5120] seed 42+b, buffer (1024,1024); golden = all_reduce -> +bias -> rms_norm; tol 4e-2
+    W = 8
+    xs = [orc.randn_bf16((b, 5120), 42 + r + b) for r in range(W)]
+    bias = orc.randn_bf16((b, 5120), 42 + b)
+    w = orc.randn_bf16((5120,), 4242 + b)
+    buf = torch.zeros(W, 1024, 1024, dtype=BF16, device=dev)
+    for r in range(1, W):
+        buf[r].view(-1)[: b * 5120].copy_(xs[r].view(-1))
+    for fn in (fused.one_shot_all_reduce_bias_rms_norm, fused.two_shot_all_reduce_bias_rms_norm):
+        y = torch.empty(b, 5120, dtype=BF16, device=dev)
+        fn(buf, xs[0].to(dev), bias.to(dev), w.to(dev), y)
+        want = orc.reduce_bias_rms_norm(torch.stack(xs), bias, w)
+        torch.testing.assert_close(y.cpu(), want, **TOL)
+        assert_one_ulp(y, want)
+        # the reference's own golden: rms_norm of the bf16-rounded all-reduce + bias
+        golden = orc.rms_norm((orc.reduce_library(torch.stack(xs)) + bias), w)
+        torch.testing.assert_close(y.cpu(), golden, rtol=4e-2, atol=4e-2)
+
+
+@pytest.mark.parametrize("W", [1, 2, 3, 4, 8, 16])
+@pytest.mark.parametrize("bias_mode", ["none", "full", "vector"])
+def test_world_sizes_and_bias_modes(dev, W, bias_mode):
+    rows, D = 9, 1000
+    stack = orc.make_stack(W, (rows, D))
+    w = orc.randn_bf16((D,), 5, 0.02, 1.0)
+    bias = {"none": None, "full": orc.randn_bf16((rows, D), 7), "vector": orc.randn_bf16((D,), 7, 0.02)}[bias_mode]
+    y = torch.empty(rows, D, dtype=BF16, device=dev)
+    fused.one_shot_all_reduce_bias_rms_norm(stack.to(dev), None, None if bias is None else bias.to(dev),
+                                            w.to(dev), y, eps=1e-5)
+    want = orc.reduce_bias_rms_norm(stack, bias, w, 1e-5)
+    torch.testing.assert_close(y.cpu(), want, **TOL)
+    assert_one_ulp(y, want)
+
+
+def test_nd_input_and_eps(dev):
+    W, B, T, D = 4, 3, 5, 512
+    stack = orc.make_stack(W, (B, T, D))
+    bias, w = orc.make_bias_weight(D)
+    y = torch.empty(B, T, D, dtype=BF16, device=dev)
+    fused.one_shot_all_reduce_bias_rms_norm(stack.to(dev), None, bias.to(dev), w.to(dev), y, eps=1e-2)
+    assert_one_ulp(y, orc.reduce_bias_rms_norm(stack, bias, w, 1e-2))
+
+
+@pytest.mark.parametrize("cfg", [(8, 256, 4096), (8, 16, 8192)])
+def test_baseline_configs_1_and_3(dev, cfg):
+    W, rows, D = cfg
+    stack = orc.make_stack(W, (rows, D), seed0=42)
+    bias, w = orc.make_bias_weight(D, 42)
+    y = torch.empty(rows, D, dtype=BF16, device=dev)
+    fused.one_shot_all_reduce_bias_rms_norm(stack.to(dev), None, bias.to(dev), w.to(dev), y, eps=1e-5)
+    want = orc.reduce_bias_rms_norm(stack, bias, w, 1e-5)
+    torch.testing.assert_close(y.cpu(), want, **TOL)
+    assert_one_ulp(y, want)
+    torch.testing.assert_close(y.cpu(), orc.reduce_bias_rms_norm_library(stack, bias, w, 1e-5), **TOL)
+    # scale invariance: x -> 2x (exact in bf16) changes nothing while mean(s^2) >> eps
+    y2 = torch.empty_like(y)
+    fused.one_shot_all_reduce_bias_rms_norm((stack * 2).to(dev), None, (bias * 2).to(dev), w.to(dev), y2, eps=1e-5)
+    torch.testing.assert_close(y2.float().cpu(), y.float().cpu(), rtol=2 ** -7, atol=1e-5)
