@@ -96,104 +96,129 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_reduce_kernel(const GemmArgs
     if (tile_m >= g.tiles_m) tile_m -= g.tiles_m;
     const int m0 = tile_m * BM, n0 = tile_n * BN;
 
-    // ---- global -> register staging ------------------------------------------
+    // ---- operand staging: global -> registers -> LDS, one 16-byte chunk per "unit" ------
+    // Per-thread byte offsets are relative to a tile base that is uniform across the
+    // workgroup (so the loads use scalar base + 32-bit vector offset addressing) and
+    // stay the same for every k-step; only the uniform base advances.
+    constexpr int NB_LD = B_NT ? B_ITERS_NT : B_BLOCKS * 8;   // 128-bit global loads of B per thread per stage
+    constexpr int NB_ST = B_NT ? B_ITERS_NT : B_BLOCKS * 4;   // B store units per thread per stage
     u32x4 a_reg[A_ITERS];
-    u32x4 b_reg[B_NT ? B_ITERS_NT : B_BLOCKS * 8];
-
-    auto load_a = [&](int k0) {
+    u32x4 b_reg[NB_LD];
+    uint32_t a_goff[A_ITERS], a_loff[A_ITERS];
+    uint32_t b_goff[B_NT ? B_ITERS_NT : B_BLOCKS], b_loff[B_NT ? B_ITERS_NT : B_BLOCKS];
+    const int ld_kc = tid & 7;        // 16-byte chunk inside a 128-byte k-row (T % 8 == 0)
+    bool nn_active = true;            // NN: this thread owns an 8x8 block of the B stage
 #pragma unroll
-        for (int i = 0; i < A_ITERS; ++i) {
-            const int c = i * T + tid;
-            const int row = c >> 3, kc = c & 7;
-            int m = m0 + row;
-            const int k = k0 + kc * 8;
+    for (int i = 0; i < A_ITERS; ++i) {
+        const int row = (i * T + tid) >> 3;
+        int m = m0 + row;
+        if (!EVEN) m = min(m, g.M - 1);
+        a_goff[i] = (uint32_t)(((int64_t)(m - m0) * g.lda + ld_kc * 8) * 2);
+        a_loff[i] = row * kRowBytes + swz(row, ld_kc) * 16;
+    }
+    if (B_NT) {
+#pragma unroll
+        for (int i = 0; i < B_ITERS_NT; ++i) {
+            const int row = (i * T + tid) >> 3;
+            int n = n0 + row;
+            if (!EVEN) n = min(n, g.N - 1);
+            b_goff[i] = (uint32_t)(((int64_t)(n - n0) * g.ldb + ld_kc * 8) * 2);
+            b_loff[i] = row * kRowBytes + swz(row, ld_kc) * 16;
+        }
+    } else {
+#pragma unroll
+        for (int i = 0; i < B_BLOCKS; ++i) {
+            const int blk = i * T + tid;
+            const int nc = blk % (BN / 8), kg = blk / (BN / 8);
+            if (BN < T && kg >= 8) nn_active = false;     // more threads than 8x8 blocks
+            int n = n0 + nc * 8;
+            if (!EVEN) n = min(n, g.N - 8);
+            b_goff[i] = (uint32_t)(((int64_t)(kg & 7) * 8 * g.ldb + (n - n0)) * 2);
+            b_loff[i] = (uint32_t)(nc | ((kg & 7) << 16));   // packed (nc, kg); expanded at the store
+        }
+    }
+    const unsigned char* a_tile = (const unsigned char*)(g.A + (int64_t)m0 * g.lda);
+    const unsigned char* b_tile = B_NT ? (const unsigned char*)(g.B + (int64_t)n0 * g.ldb)
+                                       : (const unsigned char*)(g.B + n0);
+
+    auto load_a_unit = [&](int i, int k0) {
+        const unsigned char* base = a_tile + (int64_t)k0 * 2;
+        if (EVEN) {
+            a_reg[i] = *(const u32x4*)(base + a_goff[i]);
+        } else {
+            a_reg[i] = (k0 + ld_kc * 8 < g.K) ? *(const u32x4*)(base + a_goff[i]) : u32x4{0, 0, 0, 0};
+        }
+    };
+    auto load_b_unit = [&](int u, int k0) {
+        if (B_NT) {
+            const unsigned char* base = b_tile + (int64_t)k0 * 2;
             if (EVEN) {
-                a_reg[i] = *(const u32x4*)(g.A + (int64_t)m * g.lda + k);
+                b_reg[u] = *(const u32x4*)(base + b_goff[u]);
             } else {
-                m = min(m, g.M - 1);
-                a_reg[i] = k < g.K ? *(const u32x4*)(g.A + (int64_t)m * g.lda + k) : u32x4{0, 0, 0, 0};
+                b_reg[u] = (k0 + ld_kc * 8 < g.K) ? *(const u32x4*)(base + b_goff[u]) : u32x4{0, 0, 0, 0};
+            }
+        } else {
+            const int i = u >> 3, j = u & 7;             // block i, k-row j of the 8x8 block
+            if (!nn_active) return;
+            const unsigned char* base = b_tile + ((int64_t)(k0 + j) * g.ldb) * 2;
+            if (EVEN) {
+                b_reg[u] = *(const u32x4*)(base + b_goff[i]);
+            } else {
+                const int kg = (int)(b_loff[i] >> 16);
+                b_reg[u] = (k0 + kg * 8 + j < g.K) ? *(const u32x4*)(base + b_goff[i]) : u32x4{0, 0, 0, 0};
             }
         }
     };
-    auto load_b = [&](int k0) {
+    // LDS offsets below are relative to stage 0; `st` (0 or STAGE, a power of two above every
+    // in-stage offset) selects the stage by XOR.
+    auto store_a_unit = [&](int i, uint32_t st) { *(u32x4*)(smem + (a_loff[i] ^ st)) = a_reg[i]; };
+    auto store_b_unit = [&](int u, uint32_t st) {
+        unsigned char* Bs = smem + A_STAGE;
         if (B_NT) {
-#pragma unroll
-            for (int i = 0; i < B_ITERS_NT; ++i) {
-                const int c = i * T + tid;
-                const int row = c >> 3, kc = c & 7;
-                int n = n0 + row;
-                const int k = k0 + kc * 8;
-                if (EVEN) {
-                    b_reg[i] = *(const u32x4*)(g.B + (int64_t)n * g.ldb + k);
-                } else {
-                    n = min(n, g.N - 1);
-                    b_reg[i] = k < g.K ? *(const u32x4*)(g.B + (int64_t)n * g.ldb + k) : u32x4{0, 0, 0, 0};
-                }
-            }
+            *(u32x4*)(Bs + (b_loff[u] ^ st)) = b_reg[u];
         } else {
-#pragma unroll
-            for (int i = 0; i < B_BLOCKS; ++i) {
-                const int blk = i * T + tid;
-                const int nc = blk % (BN / 8), kg = blk / (BN / 8);
-                if (BN < T && kg >= 8) continue;  // more threads than 8x8 blocks
-                int n = n0 + nc * 8;
-                if (!EVEN) n = min(n, g.N - 8);
-#pragma unroll
-                for (int j = 0; j < 8; ++j) {
-                    const int k = k0 + kg * 8 + j;
-                    if (EVEN) {
-                        b_reg[i * 8 + j] = *(const u32x4*)(g.B + (int64_t)k * g.ldb + n);
-                    } else {
-                        b_reg[i * 8 + j] =
-                            k < g.K ? *(const u32x4*)(g.B + (int64_t)k * g.ldb + n) : u32x4{0, 0, 0, 0};
-                    }
-                }
-            }
-        }
-    };
-    auto store_stage = [&](int stage) {
-        unsigned char* As = smem + stage * STAGE;
-        unsigned char* Bs = As + A_STAGE;
-#pragma unroll
-        for (int i = 0; i < A_ITERS; ++i) {
-            const int c = i * T + tid;
-            const int row = c >> 3, kc = c & 7;
-            *(u32x4*)(As + row * kRowBytes + swz(row, kc) * 16) = a_reg[i];
-        }
-        if (B_NT) {
-#pragma unroll
-            for (int i = 0; i < B_ITERS_NT; ++i) {
-                const int c = i * T + tid;
-                const int row = c >> 3, kc = c & 7;
-                *(u32x4*)(Bs + row * kRowBytes + swz(row, kc) * 16) = b_reg[i];
-            }
-        } else {
-#pragma unroll
-            for (int i = 0; i < B_BLOCKS; ++i) {
-                const int blk = i * T + tid;
-                const int nc = blk % (BN / 8), kg = blk / (BN / 8);
-                if (BN < T && kg >= 8) continue;
-                // b_reg[i*8 + j] holds row k = kg*8 + j, columns nc*8 .. nc*8+7 (two per word)
-#pragma unroll
-                for (int q = 0; q < 4; ++q) {      // word q = columns 2q, 2q+1
-                    u32x4 even, odd;               // [n = 2q][k 0..7], [n = 2q+1][k 0..7]
-                    even.x = perm_lo(b_reg[i * 8 + 1][q], b_reg[i * 8 + 0][q]);
-                    even.y = perm_lo(b_reg[i * 8 + 3][q], b_reg[i * 8 + 2][q]);
-                    even.z = perm_lo(b_reg[i * 8 + 5][q], b_reg[i * 8 + 4][q]);
-                    even.w = perm_lo(b_reg[i * 8 + 7][q], b_reg[i * 8 + 6][q]);
-                    odd.x = perm_hi(b_reg[i * 8 + 1][q], b_reg[i * 8 + 0][q]);
-                    odd.y = perm_hi(b_reg[i * 8 + 3][q], b_reg[i * 8 + 2][q]);
-                    odd.z = perm_hi(b_reg[i * 8 + 5][q], b_reg[i * 8 + 4][q]);
-                    odd.w = perm_hi(b_reg[i * 8 + 7][q], b_reg[i * 8 + 6][q]);
-                    const int r0 = nc * 8 + 2 * q, r1 = r0 + 1;
-                    *(u32x4*)(Bs + r0 * kRowBytes + swz(r0, kg) * 16) = even;
-                    *(u32x4*)(Bs + r1 * kRowBytes + swz(r1, kg) * 16) = odd;
-                }
-            }
+            // unit u = (block i, word q): columns 2q and 2q+1 of the 8x8 block, all 8 k
+            const int i = u >> 2, q = u & 3;
+            if (!nn_active) return;
+            const int nc = (int)(b_loff[i] & 0xffff), kg = (int)(b_loff[i] >> 16);
+            u32x4 even, odd;               // [n = 2q][k 0..7], [n = 2q+1][k 0..7]
+            even.x = perm_lo(b_reg[i * 8 + 1][q], b_reg[i * 8 + 0][q]);
+            even.y = perm_lo(b_reg[i * 8 + 3][q], b_reg[i * 8 + 2][q]);
+            even.z = perm_lo(b_reg[i * 8 + 5][q], b_reg[i * 8 + 4][q]);
+            even.w = perm_lo(b_reg[i * 8 + 7][q], b_reg[i * 8 + 6][q]);
+            odd.x = perm_hi(b_reg[i * 8 + 1][q], b_reg[i * 8 + 0][q]);
+            odd.y = perm_hi(b_reg[i * 8 + 3][q], b_reg[i * 8 + 2][q]);
+            odd.z = perm_hi(b_reg[i * 8 + 5][q], b_reg[i * 8 + 4][q]);
+            odd.w = perm_hi(b_reg[i * 8 + 7][q], b_reg[i * 8 + 6][q]);
+            const int r0 = nc * 8 + 2 * q, r1 = r0 + 1;
+            *(u32x4*)(Bs + ((uint32_t)(r0 * kRowBytes + swz(r0, kg) * 16) ^ st)) = even;
+            *(u32x4*)(Bs + ((uint32_t)(r1 * kRowBytes + swz(r1, kg) * 16) ^ st)) = odd;
         }
     };
 
-    // ---- main loop ----------------------------------------------------------------
+    // ---- MFMA fragments ---------------------------------------------------------------
+    // lane -> row (A) / column (B) of a 32x32 block and which 8-wide half of the 16-wide k step
+    const int frag_row = lane & 31, frag_kc = lane >> 5;
+    uint32_t fa_off[TM], fb_off[TN];   // LDS byte offset of the lane's chunk at ks = 0
+#pragma unroll
+    for (int i = 0; i < TM; ++i) {
+        const int row = wm * WTM + i * 32 + frag_row;
+        fa_off[i] = row * kRowBytes + swz(row, frag_kc) * 16;
+    }
+#pragma unroll
+    for (int j = 0; j < TN; ++j) {
+        const int row = wn * WTN + j * 32 + frag_row;
+        fb_off[j] = A_STAGE + row * kRowBytes + swz(row, frag_kc) * 16;   // A_STAGE < STAGE: survives the XOR
+    }
+    bf16x8 af[2][TM], bfr[2][TN];
+    // chunk (2*ks + kc) ^ f(row) == (kc ^ f(row)) ^ 2*ks: the k sub-step only flips address bits 5..6
+    // fa_off / fb_off carry the stage bit of the tile being computed (toggled every iteration);
+    // `other` = STAGE reads from the other stage.
+    auto read_frag = [&](int q, int ks, uint32_t other, int buf) {
+        if (q < TM) af[buf][q] = *(const bf16x8*)(smem + (fa_off[q] ^ (uint32_t)(ks << 5) ^ other));
+        else bfr[buf][q - TM] = *(const bf16x8*)(smem + (fb_off[q - TM] ^ (uint32_t)(ks << 5) ^ other));
+    };
+
     f32x16 acc[TM][TN];
 #pragma unroll
     for (int i = 0; i < TM; ++i)
@@ -202,46 +227,99 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_reduce_kernel(const GemmArgs
 #pragma unroll
             for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
 
+    // ---- software pipeline ---------------------------------------------------------------
+    // Iteration t computes tile t from LDS stage t&1 while (a) the registers holding tile
+    // t+1 (loaded from global memory during iteration t-1) are written to stage (t+1)&1 and
+    // (b) tile t+2 is loaded into those registers.  MFMA fragments are double-buffered in
+    // registers one 16-wide k sub-step ahead.  One workgroup barrier per iteration, placed
+    // before the last sub-step: by then every wave has written its part of tile t+1 and has
+    // issued (and waited for) its last reads of tile t.  All side work is spread between the
+    // MFMAs in a fixed order.
+    constexpr int NM = TM * TN, NF = TM + TN;
     const int kt_total = (g.K + BK - 1) / BK;
-    load_a(0);
-    load_b(0);
-    store_stage(0);
-    __syncthreads();
+    const int k_last = (kt_total - 1) * BK;
 
-    const int frag_row = lane & 31;   // row (A) / column (B) inside a 32x32 block
-    const int frag_kc = lane >> 5;    // which 8-wide k chunk of the 16-wide MFMA step
+#define KR_SCHED_FENCE() __builtin_amdgcn_sched_barrier(0)
+    auto mfma_step = [&](int buf, auto&& side) {
+#pragma unroll
+        for (int s = 0; s < NM; ++s) {
+            const int i = s / TN, j = s % TN;
+            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[buf][i], bfr[buf][j], acc[i][j], 0, 0, 0);
+            side(s);
+            KR_SCHED_FENCE();
+        }
+    };
+    static_assert((STAGE & (STAGE - 1)) == 0, "stage selection by XOR needs a power-of-two stage size");
+    uint32_t nxt = STAGE;   // stage (relative to stage 0) that receives tile t+1
+    auto iteration = [&](int t) {
+        const int k2 = min((t + 2) * BK, k_last);   // tile t+2, clamped: the tail re-loads the last tile
+        // sub-step 0: fragments of sub-step 1; A registers (tile t+1) -> LDS
+        mfma_step(0, [&](int s) {
+#pragma unroll
+            for (int q = s * NF / NM; q < (s + 1) * NF / NM; ++q) read_frag(q, 1, 0, 1);
+#pragma unroll
+            for (int q = s * A_ITERS / NM; q < (s + 1) * A_ITERS / NM; ++q) store_a_unit(q, nxt);
+        });
+        // sub-step 1: fragments of sub-step 2; B registers (tile t+1) -> LDS
+        mfma_step(1, [&](int s) {
+#pragma unroll
+            for (int q = s * NF / NM; q < (s + 1) * NF / NM; ++q) read_frag(q, 2, 0, 0);
+#pragma unroll
+            for (int q = s * NB_ST / NM; q < (s + 1) * NB_ST / NM; ++q) store_b_unit(q, nxt);
+        });
+        // sub-step 2: fragments of sub-step 3; global loads of A (tile t+2)
+        mfma_step(0, [&](int s) {
+#pragma unroll
+            for (int q = s * NF / NM; q < (s + 1) * NF / NM; ++q) read_frag(q, 3, 0, 1);
+#pragma unroll
+            for (int q = s * A_ITERS / NM; q < (s + 1) * A_ITERS / NM; ++q) load_a_unit(q, k2);
+        });
+        // every LDS access of this wave so far has completed; then all waves meet
+        __builtin_amdgcn_s_waitcnt(0xc07f);   // lgkmcnt(0) only: the global loads stay in flight
+        __builtin_amdgcn_s_barrier();
+        KR_SCHED_FENCE();
+        // sub-step 3: fragments of sub-step 0 of tile t+1; global loads of B (tile t+2)
+        mfma_step(1, [&](int s) {
+#pragma unroll
+            for (int q = s * NF / NM; q < (s + 1) * NF / NM; ++q) read_frag(q, 0, STAGE, 0);
+#pragma unroll
+            for (int q = s * NB_LD / NM; q < (s + 1) * NB_LD / NM; ++q) load_b_unit(q, k2);
+        });
+        // switch stages: the fragment offsets follow the tile being computed
+#pragma unroll
+        for (int i = 0; i < TM; ++i) fa_off[i] ^= STAGE;
+#pragma unroll
+        for (int j = 0; j < TN; ++j) fb_off[j] ^= STAGE;
+        nxt ^= STAGE;
+    };
 
-    for (int kt = 0; kt < kt_total; ++kt) {
-        const int cur = kt & 1;
-        const bool more = kt + 1 < kt_total;
-        if (more) {
-            load_a((kt + 1) * BK);
-            load_b((kt + 1) * BK);
-        }
-        const unsigned char* As = smem + cur * STAGE;
-        const unsigned char* Bs = As + A_STAGE;
+    // prologue: tile 0 -> stage 0, tile 1 -> registers, first fragments
 #pragma unroll
-        for (int ks = 0; ks < BK / 16; ++ks) {
-            bf16x8 af[TM], bfr[TN];
+    for (int i = 0; i < A_ITERS; ++i) load_a_unit(i, 0);
 #pragma unroll
-            for (int i = 0; i < TM; ++i) {
-                const int row = wm * WTM + i * 32 + frag_row;
-                af[i] = *(const bf16x8*)(As + row * kRowBytes + swz(row, ks * 2 + frag_kc) * 16);
-            }
+    for (int u = 0; u < NB_LD; ++u) load_b_unit(u, 0);
 #pragma unroll
-            for (int j = 0; j < TN; ++j) {
-                const int row = wn * WTN + j * 32 + frag_row;
-                bfr[j] = *(const bf16x8*)(Bs + row * kRowBytes + swz(row, ks * 2 + frag_kc) * 16);
-            }
+    for (int i = 0; i < A_ITERS; ++i) store_a_unit(i, 0);
 #pragma unroll
-            for (int i = 0; i < TM; ++i)
+    for (int u = 0; u < NB_ST; ++u) store_b_unit(u, 0);
+    {
+        const int k1 = min(BK, k_last);
 #pragma unroll
-                for (int j = 0; j < TN; ++j)
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[i], bfr[j], acc[i][j], 0, 0, 0);
-        }
-        if (more) store_stage(cur ^ 1);
-        __syncthreads();
+        for (int i = 0; i < A_ITERS; ++i) load_a_unit(i, k1);
+#pragma unroll
+        for (int u = 0; u < NB_LD; ++u) load_b_unit(u, k1);
     }
+    __builtin_amdgcn_s_waitcnt(0xc07f);
+    __builtin_amdgcn_s_barrier();
+    KR_SCHED_FENCE();
+#pragma unroll
+    for (int q = 0; q < NF; ++q) read_frag(q, 0, 0, 0);
+
+    for (int t = 0; t < kt_total; ++t) iteration(t);
+#undef KR_SCHED_FENCE
+    // the tail iterations re-load and re-store the last tile: drain everything before the
+    // LDS is reused by the epilogue
+    __syncthreads();
 
     // ---- epilogue -------------------------------------------------------------------
     // After the last barrier no wave reads the pipeline stages any more.
