@@ -19,6 +19,8 @@
 // all moved with 128-bit accesses covering whole 256-byte row segments.
 #include <stdlib.h>
 
+#include <type_traits>
+
 #include "common.h"
 
 namespace kr {
@@ -97,11 +99,12 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_reduce_kernel(const GemmArgs
     const int m0 = tile_m * BM, n0 = tile_n * BN;
 
     // ---- operand staging: global -> registers -> LDS, one 16-byte chunk per "unit" ------
-    // Per-thread byte offsets are relative to a tile base that is uniform across the
-    // workgroup (so the loads use scalar base + 32-bit vector offset addressing) and
-    // stay the same for every k-step; only the uniform base advances.
+    // Global loads are buffer loads: a wave-uniform resource descriptor (tile base), a
+    // per-thread 32-bit byte offset that never changes, and a wave-uniform scalar offset that
+    // advances with k.  No per-load address arithmetic is left in the main loop.
     constexpr int NB_LD = B_NT ? B_ITERS_NT : B_BLOCKS * 8;   // 128-bit global loads of B per thread per stage
     constexpr int NB_ST = B_NT ? B_ITERS_NT : B_BLOCKS * 4;   // B store units per thread per stage
+    constexpr uint32_t kOob = 0x80000000u;                     // offset beyond num_records: the load returns 0
     u32x4 a_reg[A_ITERS];
     u32x4 b_reg[NB_LD];
     uint32_t a_goff[A_ITERS], a_loff[A_ITERS];
@@ -123,7 +126,7 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_reduce_kernel(const GemmArgs
             int n = n0 + row;
             if (!EVEN) n = min(n, g.N - 1);
             b_goff[i] = (uint32_t)(((int64_t)(n - n0) * g.ldb + ld_kc * 8) * 2);
-            b_loff[i] = row * kRowBytes + swz(row, ld_kc) * 16;
+            b_loff[i] = A_STAGE + row * kRowBytes + swz(row, ld_kc) * 16;
         }
     } else {
 #pragma unroll
@@ -137,45 +140,43 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_reduce_kernel(const GemmArgs
             b_loff[i] = (uint32_t)(nc | ((kg & 7) << 16));   // packed (nc, kg); expanded at the store
         }
     }
-    const unsigned char* a_tile = (const unsigned char*)(g.A + (int64_t)m0 * g.lda);
-    const unsigned char* b_tile = B_NT ? (const unsigned char*)(g.B + (int64_t)n0 * g.ldb)
-                                       : (const unsigned char*)(g.B + n0);
+    // descriptors: 48-bit base, stride 0 (raw), num_records 2^31-1 bytes, 32-bit data format.
+    // Rows are clamped into the matrix above, so only the K tail needs the out-of-range path.
+    const __amdgpu_buffer_rsrc_t a_rsrc =
+        __builtin_amdgcn_make_buffer_rsrc((void*)(g.A + (int64_t)m0 * g.lda), 0, 0x7fffffff, 0x00020000);
+    const __amdgpu_buffer_rsrc_t bt_rsrc =
+        __builtin_amdgcn_make_buffer_rsrc((void*)(g.B + (int64_t)n0 * g.ldb), 0, 0x7fffffff, 0x00020000);
 
     auto load_a_unit = [&](int i, int k0) {
-        const unsigned char* base = a_tile + (int64_t)k0 * 2;
-        if (EVEN) {
-            a_reg[i] = *(const u32x4*)(base + a_goff[i]);
-        } else {
-            a_reg[i] = (k0 + ld_kc * 8 < g.K) ? *(const u32x4*)(base + a_goff[i]) : u32x4{0, 0, 0, 0};
-        }
+        uint32_t off = a_goff[i];
+        if (!EVEN && k0 + ld_kc * 8 >= g.K) off = kOob;
+        a_reg[i] = __builtin_amdgcn_raw_buffer_load_b128(a_rsrc, off, k0 * 2, 0);
     };
     auto load_b_unit = [&](int u, int k0) {
         if (B_NT) {
-            const unsigned char* base = b_tile + (int64_t)k0 * 2;
-            if (EVEN) {
-                b_reg[u] = *(const u32x4*)(base + b_goff[u]);
-            } else {
-                b_reg[u] = (k0 + ld_kc * 8 < g.K) ? *(const u32x4*)(base + b_goff[u]) : u32x4{0, 0, 0, 0};
-            }
+            uint32_t off = b_goff[u];
+            if (!EVEN && k0 + ld_kc * 8 >= g.K) off = kOob;
+            b_reg[u] = __builtin_amdgcn_raw_buffer_load_b128(bt_rsrc, off, k0 * 2, 0);
         } else {
             const int i = u >> 3, j = u & 7;             // block i, k-row j of the 8x8 block
             if (!nn_active) return;
-            const unsigned char* base = b_tile + ((int64_t)(k0 + j) * g.ldb) * 2;
-            if (EVEN) {
-                b_reg[u] = *(const u32x4*)(base + b_goff[i]);
-            } else {
-                const int kg = (int)(b_loff[i] >> 16);
-                b_reg[u] = (k0 + kg * 8 + j < g.K) ? *(const u32x4*)(base + b_goff[i]) : u32x4{0, 0, 0, 0};
-            }
+            // re-based on the k-row so that the scalar offset stays small for any matrix size
+            const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc(
+                (void*)(g.B + (int64_t)(k0 + j) * g.ldb + n0), 0, 0x7fffffff, 0x00020000);
+            uint32_t off = b_goff[i];
+            if (!EVEN && k0 + (int)(b_loff[i] >> 16) * 8 + j >= g.K) off = kOob;
+            b_reg[u] = __builtin_amdgcn_raw_buffer_load_b128(rs, off, 0, 0);
         }
     };
-    // LDS offsets below are relative to stage 0; `st` (0 or STAGE, a power of two above every
-    // in-stage offset) selects the stage by XOR.
-    auto store_a_unit = [&](int i, uint32_t st) { *(u32x4*)(smem + (a_loff[i] ^ st)) = a_reg[i]; };
+    // LDS is addressed by raw byte offsets: this kernel declares no static LDS, so its dynamic
+    // array starts at LDS address 0.  Offsets are relative to stage 0; `st` (0 or STAGE, a power
+    // of two above every in-stage offset) selects the stage by XOR.
+    typedef __attribute__((address_space(3))) u32x4* lds_u32x4;
+    typedef const __attribute__((address_space(3))) bf16x8* lds_frag;
+    auto store_a_unit = [&](int i, uint32_t st) { *(lds_u32x4)(a_loff[i] ^ st) = a_reg[i]; };
     auto store_b_unit = [&](int u, uint32_t st) {
-        unsigned char* Bs = smem + A_STAGE;
         if (B_NT) {
-            *(u32x4*)(Bs + (b_loff[u] ^ st)) = b_reg[u];
+            *(lds_u32x4)(b_loff[u] ^ st) = b_reg[u];
         } else {
             // unit u = (block i, word q): columns 2q and 2q+1 of the 8x8 block, all 8 k
             const int i = u >> 2, q = u & 3;
@@ -191,8 +192,8 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_reduce_kernel(const GemmArgs
             odd.z = perm_hi(b_reg[i * 8 + 5][q], b_reg[i * 8 + 4][q]);
             odd.w = perm_hi(b_reg[i * 8 + 7][q], b_reg[i * 8 + 6][q]);
             const int r0 = nc * 8 + 2 * q, r1 = r0 + 1;
-            *(u32x4*)(Bs + ((uint32_t)(r0 * kRowBytes + swz(r0, kg) * 16) ^ st)) = even;
-            *(u32x4*)(Bs + ((uint32_t)(r1 * kRowBytes + swz(r1, kg) * 16) ^ st)) = odd;
+            *(lds_u32x4)((uint32_t)(A_STAGE + r0 * kRowBytes + swz(r0, kg) * 16) ^ st) = even;
+            *(lds_u32x4)((uint32_t)(A_STAGE + r1 * kRowBytes + swz(r1, kg) * 16) ^ st) = odd;
         }
     };
 
@@ -215,8 +216,8 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_reduce_kernel(const GemmArgs
     // fa_off / fb_off carry the stage bit of the tile being computed (toggled every iteration);
     // `other` = STAGE reads from the other stage.
     auto read_frag = [&](int q, int ks, uint32_t other, int buf) {
-        if (q < TM) af[buf][q] = *(const bf16x8*)(smem + (fa_off[q] ^ (uint32_t)(ks << 5) ^ other));
-        else bfr[buf][q - TM] = *(const bf16x8*)(smem + (fb_off[q - TM] ^ (uint32_t)(ks << 5) ^ other));
+        if (q < TM) af[buf][q] = *(lds_frag)(fa_off[q] ^ (uint32_t)(ks << 5) ^ other);
+        else bfr[buf][q - TM] = *(lds_frag)(fb_off[q - TM] ^ (uint32_t)(ks << 5) ^ other);
     };
 
     f32x16 acc[TM][TN];
@@ -240,51 +241,60 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_reduce_kernel(const GemmArgs
     const int k_last = (kt_total - 1) * BK;
 
 #define KR_SCHED_FENCE() __builtin_amdgcn_sched_barrier(0)
-    auto mfma_step = [&](int buf, auto&& side) {
+    // Side work of one iteration, in the order it is issued: A units, then B units; a unit is
+    // "write the registers of tile t+1 to LDS, then re-fill them with tile t+2" (so those
+    // loads have a whole iteration to land).  Row-major B consumes the 8 registers of a block
+    // in 4 store units before the block is re-loaded.  The jobs are spread evenly over the MFMA
+    // slots of sub-steps 0..2; sub-step 3 follows the barrier.
+    constexpr int NJ = A_ITERS + (B_NT ? NB_ST : NB_ST + NB_LD);
+    constexpr int NSL = 3 * NM;
+    uint32_t nxt = STAGE;   // stage (relative to stage 0) that receives tile t+1
+    static_assert((STAGE & (STAGE - 1)) == 0, "stage selection by XOR needs a power-of-two stage size");
+    auto staging_job = [&](int j, int k2) {
+        if (j < A_ITERS) {
+            store_a_unit(j, nxt);
+            load_a_unit(j, k2);
+        } else if (B_NT) {
+            store_b_unit(j - A_ITERS, nxt);
+            load_b_unit(j - A_ITERS, k2);
+        } else if (j - A_ITERS < NB_ST) {
+            store_b_unit(j - A_ITERS, nxt);
+        } else {
+            load_b_unit(j - A_ITERS - NB_ST, k2);
+        }
+    };
+    // one 16-wide k sub-step: NM MFMAs on fragment buffer `buf`; after each MFMA the fragment
+    // reads of the next sub-step (into the other buffer) and the staging jobs of that slot
+    auto mfma_step = [&](auto ks_c, int k2) {
+        constexpr int ks = decltype(ks_c)::value;
+        constexpr int buf = ks & 1;
+        constexpr bool staging = ks < 3;
 #pragma unroll
         for (int s = 0; s < NM; ++s) {
             const int i = s / TN, j = s % TN;
             acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[buf][i], bfr[buf][j], acc[i][j], 0, 0, 0);
-            side(s);
+#pragma unroll
+            for (int q = s * NF / NM; q < (s + 1) * NF / NM; ++q)
+                read_frag(q, (ks + 1) & 3, ks == 3 ? STAGE : 0, buf ^ 1);
+            if constexpr (staging) {
+                const int slot = ks * NM + s;
+#pragma unroll
+                for (int jj = slot * NJ / NSL; jj < (slot + 1) * NJ / NSL; ++jj) staging_job(jj, k2);
+            }
             KR_SCHED_FENCE();
         }
     };
-    static_assert((STAGE & (STAGE - 1)) == 0, "stage selection by XOR needs a power-of-two stage size");
-    uint32_t nxt = STAGE;   // stage (relative to stage 0) that receives tile t+1
     auto iteration = [&](int t) {
         const int k2 = min((t + 2) * BK, k_last);   // tile t+2, clamped: the tail re-loads the last tile
-        // sub-step 0: fragments of sub-step 1; A registers (tile t+1) -> LDS
-        mfma_step(0, [&](int s) {
-#pragma unroll
-            for (int q = s * NF / NM; q < (s + 1) * NF / NM; ++q) read_frag(q, 1, 0, 1);
-#pragma unroll
-            for (int q = s * A_ITERS / NM; q < (s + 1) * A_ITERS / NM; ++q) store_a_unit(q, nxt);
-        });
-        // sub-step 1: fragments of sub-step 2; B registers (tile t+1) -> LDS
-        mfma_step(1, [&](int s) {
-#pragma unroll
-            for (int q = s * NF / NM; q < (s + 1) * NF / NM; ++q) read_frag(q, 2, 0, 0);
-#pragma unroll
-            for (int q = s * NB_ST / NM; q < (s + 1) * NB_ST / NM; ++q) store_b_unit(q, nxt);
-        });
-        // sub-step 2: fragments of sub-step 3; global loads of A (tile t+2)
-        mfma_step(0, [&](int s) {
-#pragma unroll
-            for (int q = s * NF / NM; q < (s + 1) * NF / NM; ++q) read_frag(q, 3, 0, 1);
-#pragma unroll
-            for (int q = s * A_ITERS / NM; q < (s + 1) * A_ITERS / NM; ++q) load_a_unit(q, k2);
-        });
+        mfma_step(std::integral_constant<int, 0>{}, k2);
+        mfma_step(std::integral_constant<int, 1>{}, k2);
+        mfma_step(std::integral_constant<int, 2>{}, k2);
         // every LDS access of this wave so far has completed; then all waves meet
         __builtin_amdgcn_s_waitcnt(0xc07f);   // lgkmcnt(0) only: the global loads stay in flight
         __builtin_amdgcn_s_barrier();
         KR_SCHED_FENCE();
-        // sub-step 3: fragments of sub-step 0 of tile t+1; global loads of B (tile t+2)
-        mfma_step(1, [&](int s) {
-#pragma unroll
-            for (int q = s * NF / NM; q < (s + 1) * NF / NM; ++q) read_frag(q, 0, STAGE, 0);
-#pragma unroll
-            for (int q = s * NB_LD / NM; q < (s + 1) * NB_LD / NM; ++q) load_b_unit(q, k2);
-        });
+        // sub-step 3 reads the fragments of sub-step 0 of tile t+1
+        mfma_step(std::integral_constant<int, 3>{}, k2);
         // switch stages: the fragment offsets follow the tile being computed
 #pragma unroll
         for (int i = 0; i < TM; ++i) fa_off[i] ^= STAGE;
