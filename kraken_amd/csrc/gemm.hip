@@ -105,8 +105,10 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_reduce_kernel(const GemmArgs
     constexpr int NB_LD = B_NT ? B_ITERS_NT : B_BLOCKS * 8;   // 128-bit global loads of B per thread per stage
     constexpr int NB_ST = B_NT ? B_ITERS_NT : B_BLOCKS * 4;   // B store units per thread per stage
     constexpr uint32_t kOob = 0x80000000u;                     // offset beyond num_records: the load returns 0
-    u32x4 a_reg[A_ITERS];
-    u32x4 b_reg[NB_LD];
+    // two register sets: set (t & 1) holds tile t+1 during iteration t and is re-filled with
+    // tile t+3, so a global load has two iterations to land
+    u32x4 a_reg[2][A_ITERS];
+    u32x4 b_reg[2][NB_LD];
     uint32_t a_goff[A_ITERS], a_loff[A_ITERS];
     uint32_t b_goff[B_NT ? B_ITERS_NT : B_BLOCKS], b_loff[B_NT ? B_ITERS_NT : B_BLOCKS];
     const int ld_kc = tid & 7;        // 16-byte chunk inside a 128-byte k-row (T % 8 == 0)
@@ -147,25 +149,25 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_reduce_kernel(const GemmArgs
     const __amdgpu_buffer_rsrc_t bt_rsrc =
         __builtin_amdgcn_make_buffer_rsrc((void*)(g.B + (int64_t)n0 * g.ldb), 0, 0x7fffffff, 0x00020000);
 
-    auto load_a_unit = [&](int i, int k0) {
+    auto load_a_unit = [&](int rs, int i, int k0) {
         uint32_t off = a_goff[i];
         if (!EVEN && k0 + ld_kc * 8 >= g.K) off = kOob;
-        a_reg[i] = __builtin_amdgcn_raw_buffer_load_b128(a_rsrc, off, k0 * 2, 0);
+        a_reg[rs][i] = __builtin_amdgcn_raw_buffer_load_b128(a_rsrc, off, k0 * 2, 0);
     };
-    auto load_b_unit = [&](int u, int k0) {
+    auto load_b_unit = [&](int rs, int u, int k0) {
         if (B_NT) {
             uint32_t off = b_goff[u];
             if (!EVEN && k0 + ld_kc * 8 >= g.K) off = kOob;
-            b_reg[u] = __builtin_amdgcn_raw_buffer_load_b128(bt_rsrc, off, k0 * 2, 0);
+            b_reg[rs][u] = __builtin_amdgcn_raw_buffer_load_b128(bt_rsrc, off, k0 * 2, 0);
         } else {
             const int i = u >> 3, j = u & 7;             // block i, k-row j of the 8x8 block
             if (!nn_active) return;
             // re-based on the k-row so that the scalar offset stays small for any matrix size
-            const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc(
+            const __amdgpu_buffer_rsrc_t brs = __builtin_amdgcn_make_buffer_rsrc(
                 (void*)(g.B + (int64_t)(k0 + j) * g.ldb + n0), 0, 0x7fffffff, 0x00020000);
             uint32_t off = b_goff[i];
             if (!EVEN && k0 + (int)(b_loff[i] >> 16) * 8 + j >= g.K) off = kOob;
-            b_reg[u] = __builtin_amdgcn_raw_buffer_load_b128(rs, off, 0, 0);
+            b_reg[rs][u] = __builtin_amdgcn_raw_buffer_load_b128(brs, off, 0, 0);
         }
     };
     // LDS is addressed by raw byte offsets: this kernel declares no static LDS, so its dynamic
@@ -173,24 +175,24 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_reduce_kernel(const GemmArgs
     // of two above every in-stage offset) selects the stage by XOR.
     typedef __attribute__((address_space(3))) u32x4* lds_u32x4;
     typedef const __attribute__((address_space(3))) bf16x8* lds_frag;
-    auto store_a_unit = [&](int i, uint32_t st) { *(lds_u32x4)(a_loff[i] ^ st) = a_reg[i]; };
-    auto store_b_unit = [&](int u, uint32_t st) {
+    auto store_a_unit = [&](int rs, int i, uint32_t st) { *(lds_u32x4)(a_loff[i] ^ st) = a_reg[rs][i]; };
+    auto store_b_unit = [&](int rs, int u, uint32_t st) {
         if (B_NT) {
-            *(lds_u32x4)(b_loff[u] ^ st) = b_reg[u];
+            *(lds_u32x4)(b_loff[u] ^ st) = b_reg[rs][u];
         } else {
             // unit u = (block i, word q): columns 2q and 2q+1 of the 8x8 block, all 8 k
             const int i = u >> 2, q = u & 3;
             if (!nn_active) return;
             const int nc = (int)(b_loff[i] & 0xffff), kg = (int)(b_loff[i] >> 16);
             u32x4 even, odd;               // [n = 2q][k 0..7], [n = 2q+1][k 0..7]
-            even.x = perm_lo(b_reg[i * 8 + 1][q], b_reg[i * 8 + 0][q]);
-            even.y = perm_lo(b_reg[i * 8 + 3][q], b_reg[i * 8 + 2][q]);
-            even.z = perm_lo(b_reg[i * 8 + 5][q], b_reg[i * 8 + 4][q]);
-            even.w = perm_lo(b_reg[i * 8 + 7][q], b_reg[i * 8 + 6][q]);
-            odd.x = perm_hi(b_reg[i * 8 + 1][q], b_reg[i * 8 + 0][q]);
-            odd.y = perm_hi(b_reg[i * 8 + 3][q], b_reg[i * 8 + 2][q]);
-            odd.z = perm_hi(b_reg[i * 8 + 5][q], b_reg[i * 8 + 4][q]);
-            odd.w = perm_hi(b_reg[i * 8 + 7][q], b_reg[i * 8 + 6][q]);
+            even.x = perm_lo(b_reg[rs][i * 8 + 1][q], b_reg[rs][i * 8 + 0][q]);
+            even.y = perm_lo(b_reg[rs][i * 8 + 3][q], b_reg[rs][i * 8 + 2][q]);
+            even.z = perm_lo(b_reg[rs][i * 8 + 5][q], b_reg[rs][i * 8 + 4][q]);
+            even.w = perm_lo(b_reg[rs][i * 8 + 7][q], b_reg[rs][i * 8 + 6][q]);
+            odd.x = perm_hi(b_reg[rs][i * 8 + 1][q], b_reg[rs][i * 8 + 0][q]);
+            odd.y = perm_hi(b_reg[rs][i * 8 + 3][q], b_reg[rs][i * 8 + 2][q]);
+            odd.z = perm_hi(b_reg[rs][i * 8 + 5][q], b_reg[rs][i * 8 + 4][q]);
+            odd.w = perm_hi(b_reg[rs][i * 8 + 7][q], b_reg[rs][i * 8 + 6][q]);
             const int r0 = nc * 8 + 2 * q, r1 = r0 + 1;
             *(lds_u32x4)((uint32_t)(A_STAGE + r0 * kRowBytes + swz(r0, kg) * 16) ^ st) = even;
             *(lds_u32x4)((uint32_t)(A_STAGE + r1 * kRowBytes + swz(r1, kg) * 16) ^ st) = odd;
@@ -250,23 +252,24 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_reduce_kernel(const GemmArgs
     constexpr int NSL = 3 * NM;
     uint32_t nxt = STAGE;   // stage (relative to stage 0) that receives tile t+1
     static_assert((STAGE & (STAGE - 1)) == 0, "stage selection by XOR needs a power-of-two stage size");
-    auto staging_job = [&](int j, int k2) {
+    auto staging_job = [&](int rs, int j, int k2) {
         if (j < A_ITERS) {
-            store_a_unit(j, nxt);
-            load_a_unit(j, k2);
+            store_a_unit(rs, j, nxt);
+            load_a_unit(rs, j, k2);
         } else if (B_NT) {
-            store_b_unit(j - A_ITERS, nxt);
-            load_b_unit(j - A_ITERS, k2);
+            store_b_unit(rs, j - A_ITERS, nxt);
+            load_b_unit(rs, j - A_ITERS, k2);
         } else if (j - A_ITERS < NB_ST) {
-            store_b_unit(j - A_ITERS, nxt);
+            store_b_unit(rs, j - A_ITERS, nxt);
         } else {
-            load_b_unit(j - A_ITERS - NB_ST, k2);
+            load_b_unit(rs, j - A_ITERS - NB_ST, k2);
         }
     };
     // one 16-wide k sub-step: NM MFMAs on fragment buffer `buf`; after each MFMA the fragment
     // reads of the next sub-step (into the other buffer) and the staging jobs of that slot
-    auto mfma_step = [&](auto ks_c, int k2) {
+    auto mfma_step = [&](auto ks_c, auto rs_c, int k2) {
         constexpr int ks = decltype(ks_c)::value;
+        constexpr int rs = decltype(rs_c)::value;
         constexpr int buf = ks & 1;
         constexpr bool staging = ks < 3;
 #pragma unroll
@@ -279,22 +282,36 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_reduce_kernel(const GemmArgs
             if constexpr (staging) {
                 const int slot = ks * NM + s;
 #pragma unroll
-                for (int jj = slot * NJ / NSL; jj < (slot + 1) * NJ / NSL; ++jj) staging_job(jj, k2);
+                for (int jj = slot * NJ / NSL; jj < (slot + 1) * NJ / NSL; ++jj) staging_job(rs, jj, k2);
             }
             KR_SCHED_FENCE();
         }
     };
-    auto iteration = [&](int t) {
-        const int k2 = min((t + 2) * BK, k_last);   // tile t+2, clamped: the tail re-loads the last tile
-        mfma_step(std::integral_constant<int, 0>{}, k2);
-        mfma_step(std::integral_constant<int, 1>{}, k2);
-        mfma_step(std::integral_constant<int, 2>{}, k2);
+    auto iteration = [&](int t, auto rs_c) {
+        const int k2 = min((t + 3) * BK, k_last);   // tile t+3, clamped: the tail re-loads the last tile
+        // The LDS offsets flip between the two stages every iteration.  Hide their values from
+        // the optimiser here, or it pre-computes every (stage, sub-step) address variant outside
+        // the loop and runs out of registers; the XORs it keeps inside are free next to the MFMAs.
+#pragma unroll
+        for (int i = 0; i < TM; ++i) asm volatile("" : "+v"(fa_off[i]));
+#pragma unroll
+        for (int j = 0; j < TN; ++j) asm volatile("" : "+v"(fb_off[j]));
+#pragma unroll
+        for (int i = 0; i < A_ITERS; ++i) asm volatile("" : "+v"(a_loff[i]));
+        if (B_NT) {
+#pragma unroll
+            for (int i = 0; i < B_ITERS_NT; ++i) asm volatile("" : "+v"(b_loff[i]));
+        }
+        asm volatile("" : "+s"(nxt));
+        mfma_step(std::integral_constant<int, 0>{}, rs_c, k2);
+        mfma_step(std::integral_constant<int, 1>{}, rs_c, k2);
+        mfma_step(std::integral_constant<int, 2>{}, rs_c, k2);
         // every LDS access of this wave so far has completed; then all waves meet
         __builtin_amdgcn_s_waitcnt(0xc07f);   // lgkmcnt(0) only: the global loads stay in flight
         __builtin_amdgcn_s_barrier();
         KR_SCHED_FENCE();
         // sub-step 3 reads the fragments of sub-step 0 of tile t+1
-        mfma_step(std::integral_constant<int, 3>{}, k2);
+        mfma_step(std::integral_constant<int, 3>{}, rs_c, k2);
         // switch stages: the fragment offsets follow the tile being computed
 #pragma unroll
         for (int i = 0; i < TM; ++i) fa_off[i] ^= STAGE;
@@ -303,21 +320,25 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_reduce_kernel(const GemmArgs
         nxt ^= STAGE;
     };
 
-    // prologue: tile 0 -> stage 0, tile 1 -> registers, first fragments
+    // prologue: tile 0 -> stage 0, tiles 1 and 2 -> the two register sets, first fragments
 #pragma unroll
-    for (int i = 0; i < A_ITERS; ++i) load_a_unit(i, 0);
+    for (int i = 0; i < A_ITERS; ++i) load_a_unit(0, i, 0);
 #pragma unroll
-    for (int u = 0; u < NB_LD; ++u) load_b_unit(u, 0);
+    for (int u = 0; u < NB_LD; ++u) load_b_unit(0, u, 0);
 #pragma unroll
-    for (int i = 0; i < A_ITERS; ++i) store_a_unit(i, 0);
+    for (int i = 0; i < A_ITERS; ++i) store_a_unit(0, i, 0);
 #pragma unroll
-    for (int u = 0; u < NB_ST; ++u) store_b_unit(u, 0);
+    for (int u = 0; u < NB_ST; ++u) store_b_unit(0, u, 0);
     {
-        const int k1 = min(BK, k_last);
+        const int k1 = min(BK, k_last), k2 = min(2 * BK, k_last);
 #pragma unroll
-        for (int i = 0; i < A_ITERS; ++i) load_a_unit(i, k1);
+        for (int i = 0; i < A_ITERS; ++i) load_a_unit(0, i, k1);
 #pragma unroll
-        for (int u = 0; u < NB_LD; ++u) load_b_unit(u, k1);
+        for (int u = 0; u < NB_LD; ++u) load_b_unit(0, u, k1);
+#pragma unroll
+        for (int i = 0; i < A_ITERS; ++i) load_a_unit(1, i, k2);
+#pragma unroll
+        for (int u = 0; u < NB_LD; ++u) load_b_unit(1, u, k2);
     }
     __builtin_amdgcn_s_waitcnt(0xc07f);
     __builtin_amdgcn_s_barrier();
@@ -325,7 +346,14 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_reduce_kernel(const GemmArgs
 #pragma unroll
     for (int q = 0; q < NF; ++q) read_frag(q, 0, 0, 0);
 
-    for (int t = 0; t < kt_total; ++t) iteration(t);
+    // branch-free body (a conditional second half would put 256 live accumulators through
+    // control-flow merges); an odd last tile is peeled
+    int t = 0;
+    for (; t + 1 < kt_total; t += 2) {
+        iteration(t, std::integral_constant<int, 0>{});
+        iteration(t + 1, std::integral_constant<int, 1>{});
+    }
+    if (t < kt_total) iteration(t, std::integral_constant<int, 0>{});
 #undef KR_SCHED_FENCE
     // the tail iterations re-load and re-store the last tile: drain everything before the
     // LDS is reused by the epilogue
