@@ -45,7 +45,7 @@ struct GemmArgs {
 
 constexpr int BK = 64;            // k extent of one LDS stage
 constexpr int kRowBytes = BK * 2; // 128-byte LDS rows
-constexpr int kGroupM = 4;        // M tiles per scheduling group
+constexpr int kGroupN = 4;        // column panels per scheduling group
 constexpr int kXcds = 8;
 
 // 16-byte chunk swizzle inside a 128-byte LDS row
@@ -84,16 +84,24 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_reduce_kernel(const GemmArgs
     const int wave = tid >> 6;
     const int wm = wave / WN, wn = wave % WN;
 
-    // ---- tile schedule: XCD-contiguous, grouped along M, rotated by the pivot
+    // ---- tile schedule -------------------------------------------------------------------
+    // Workgroups are dealt round-robin to the 8 XCDs (each with its own L2), so workgroup ids
+    // are first re-numbered to give every XCD a contiguous range of tiles.  Tiles are then
+    // ordered in groups of kGroupN column panels, M fastest in steps of kGroupN columns: the
+    // ~32 tiles an XCD runs at a time form an 8 x 4 block that shares 8 A panels and 4 B
+    // panels through its L2, and every XCD works on all row bands -- the rows of the reduce
+    // band (whose tiles also stream the peers' partial sums) are spread over all XCDs
+    // instead of landing on one.  The M order is rotated by the pivot, so the band's (or the
+    // local shard's) tiles are the first ones of every XCD.
     int pid = blockIdx.x;
     const int ntiles = g.tiles_m * g.tiles_n;
     if (ntiles % kXcds == 0) pid = (pid % kXcds) * (ntiles / kXcds) + pid / kXcds;
-    const int per_group = kGroupM * g.tiles_n;
+    const int per_group = kGroupN * g.tiles_m;
     const int group = pid / per_group;
-    const int first_m = group * kGroupM;
-    const int gsz = min(g.tiles_m - first_m, kGroupM);
-    int tile_m = first_m + (pid % per_group) % gsz;
-    const int tile_n = (pid % per_group) / gsz;
+    const int first_n = group * kGroupN;
+    const int gsz = min(g.tiles_n - first_n, kGroupN);
+    const int tile_n = first_n + (pid % per_group) % gsz;
+    int tile_m = (pid % per_group) / gsz;
     tile_m += g.pivot_tiles;
     if (tile_m >= g.tiles_m) tile_m -= g.tiles_m;
     const int m0 = tile_m * BM, n0 = tile_n * BN;
@@ -175,10 +183,10 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_reduce_kernel(const GemmArgs
     // of two above every in-stage offset) selects the stage by XOR.
     typedef __attribute__((address_space(3))) u32x4* lds_u32x4;
     typedef const __attribute__((address_space(3))) bf16x8* lds_frag;
-    auto store_a_unit = [&](int rs, int i, uint32_t st) { *(lds_u32x4)(a_loff[i] ^ st) = a_reg[rs][i]; };
+    auto store_a_unit = [&](int rs, int i, uint32_t st) { *(lds_u32x4)(size_t)(a_loff[i] ^ st) = a_reg[rs][i]; };
     auto store_b_unit = [&](int rs, int u, uint32_t st) {
         if (B_NT) {
-            *(lds_u32x4)(b_loff[u] ^ st) = b_reg[rs][u];
+            *(lds_u32x4)(size_t)(b_loff[u] ^ st) = b_reg[rs][u];
         } else {
             // unit u = (block i, word q): columns 2q and 2q+1 of the 8x8 block, all 8 k
             const int i = u >> 2, q = u & 3;
@@ -194,8 +202,8 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_reduce_kernel(const GemmArgs
             odd.z = perm_hi(b_reg[rs][i * 8 + 5][q], b_reg[rs][i * 8 + 4][q]);
             odd.w = perm_hi(b_reg[rs][i * 8 + 7][q], b_reg[rs][i * 8 + 6][q]);
             const int r0 = nc * 8 + 2 * q, r1 = r0 + 1;
-            *(lds_u32x4)((uint32_t)(A_STAGE + r0 * kRowBytes + swz(r0, kg) * 16) ^ st) = even;
-            *(lds_u32x4)((uint32_t)(A_STAGE + r1 * kRowBytes + swz(r1, kg) * 16) ^ st) = odd;
+            *(lds_u32x4)(size_t)((uint32_t)(A_STAGE + r0 * kRowBytes + swz(r0, kg) * 16) ^ st) = even;
+            *(lds_u32x4)(size_t)((uint32_t)(A_STAGE + r1 * kRowBytes + swz(r1, kg) * 16) ^ st) = odd;
         }
     };
 
@@ -218,8 +226,8 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_reduce_kernel(const GemmArgs
     // fa_off / fb_off carry the stage bit of the tile being computed (toggled every iteration);
     // `other` = STAGE reads from the other stage.
     auto read_frag = [&](int q, int ks, uint32_t other, int buf) {
-        if (q < TM) af[buf][q] = *(lds_frag)(fa_off[q] ^ (uint32_t)(ks << 5) ^ other);
-        else bfr[buf][q - TM] = *(lds_frag)(fb_off[q - TM] ^ (uint32_t)(ks << 5) ^ other);
+        if (q < TM) af[buf][q] = *(lds_frag)(size_t)(fa_off[q] ^ (uint32_t)(ks << 5) ^ other);
+        else bfr[buf][q - TM] = *(lds_frag)(size_t)(fb_off[q - TM] ^ (uint32_t)(ks << 5) ^ other);
     };
 
     f32x16 acc[TM][TN];
@@ -253,6 +261,9 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_reduce_kernel(const GemmArgs
     uint32_t nxt = STAGE;   // stage (relative to stage 0) that receives tile t+1
     static_assert((STAGE & (STAGE - 1)) == 0, "stage selection by XOR needs a power-of-two stage size");
     auto staging_job = [&](int rs, int j, int k2) {
+#ifdef KR_EXP_NOSTAGING
+        return;
+#endif
         if (j < A_ITERS) {
             store_a_unit(rs, j, nxt);
             load_a_unit(rs, j, k2);
@@ -308,7 +319,9 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_reduce_kernel(const GemmArgs
         mfma_step(std::integral_constant<int, 2>{}, rs_c, k2);
         // every LDS access of this wave so far has completed; then all waves meet
         __builtin_amdgcn_s_waitcnt(0xc07f);   // lgkmcnt(0) only: the global loads stay in flight
+#ifndef KR_EXP_NOBARRIER
         __builtin_amdgcn_s_barrier();
+#endif
         KR_SCHED_FENCE();
         // sub-step 3 reads the fragments of sub-step 0 of tile t+1
         mfma_step(std::integral_constant<int, 3>{}, rs_c, k2);
@@ -360,11 +373,21 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_reduce_kernel(const GemmArgs
     __syncthreads();
 
     // ---- epilogue -------------------------------------------------------------------
-    // After the last barrier no wave reads the pipeline stages any more.
+    // After the barrier above no wave reads the pipeline stages any more, and from here on
+    // every wave touches only its own LDS patch, so no further workgroup barrier is needed
+    // (LDS requests of one wave are served in order).  Per 32-row slab the accumulators are
+    // written to the patch in MFMA layout and read back as row-contiguous 8-element chunks.
+    // The partial sums of the other ranks are fetched kPeerGroup peers x kChunkBatch chunks at
+    // a time, all loads issued before the first add, so a band tile keeps dozens of 1 KiB
+    // wave-loads in flight instead of waiting for one HBM round trip per peer.
     float* patch = (float*)(smem + wave * EP_WAVE);
     constexpr int CPR = WTN / 8;            // 8-element chunks per patch row
     constexpr int EP_ITERS = 32 * CPR / 64; // chunks per lane per 32-row slab
+    constexpr int kChunkBatch = BM >= 256 ? 4 : 2;   // the small tile keeps its register count low (occupancy)
+    constexpr int kPeerGroup = 8;
+    static_assert(2 * kPeerGroup >= KR_MAX_WORLD - 1, "two peer groups must cover every world size");
     const int band_lo = g.band_row0, band_hi = g.band_row0 + g.band_rows;
+    const int lane_r = lane / CPR, lane_cc = lane % CPR;   // chunk (it*64 + lane): row it*(64/CPR) + lane_r
 
 #pragma unroll
     for (int i = 0; i < TM; ++i) {
@@ -376,36 +399,77 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_reduce_kernel(const GemmArgs
                 const int r = 8 * (v >> 2) + 4 * (lane >> 5) + (v & 3);
                 patch[r * EP_LD + j * 32 + (lane & 31)] = acc[i][j][v];
             }
-        __syncthreads();
+        // keep the scheduler from pulling the accumulator reads of later slabs (256 registers
+        // in all) ahead of this point
+        __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-        for (int it = 0; it < EP_ITERS; ++it) {
-            const int c = it * 64 + lane;
-            const int r = c / CPR, cc = c % CPR;
-            const int m = m0 + wm * WTM + i * 32 + r;
-            const int n = n0 + wn * WTN + cc * 8;
-            if (!EVEN && (m >= g.M || n >= g.N)) continue;
-            float f[8];
-            const f32x4 lo = *(const f32x4*)(patch + r * EP_LD + cc * 8);
-            const f32x4 hi = *(const f32x4*)(patch + r * EP_LD + cc * 8 + 4);
-            f[0] = lo.x; f[1] = lo.y; f[2] = lo.z; f[3] = lo.w;
-            f[4] = hi.x; f[5] = hi.y; f[6] = hi.z; f[7] = hi.w;
-            if (m >= band_lo && m < band_hi) {
-                const int64_t off = (int64_t)(m - band_lo) * g.N + n;
-                for (int p = 0; p < g.n_peers; ++p)
-                    add8(ld_stream((const u32x4*)(g.peers + p * g.peers_stride + off)), f);
-                if (g.bias != nullptr) add8(*(const u32x4*)(g.bias + n), f);
-                if (g.out_is_fp32) {
-                    float* o = (float*)g.out + off;
-                    *(f32x4*)o = f32x4{f[0], f[1], f[2], f[3]};
-                    *(f32x4*)(o + 4) = f32x4{f[4], f[5], f[6], f[7]};
-                } else {
-                    st_stream((u32x4*)((uint16_t*)g.out + off), pack8(f));
-                }
-            } else if (g.c_full != nullptr) {
-                st_stream((u32x4*)(g.c_full + (int64_t)m * g.N + n), pack8(f));
+        for (int b0 = 0; b0 < EP_ITERS; b0 += kChunkBatch) {
+            float f[kChunkBatch][8];
+            int64_t off[kChunkBatch];
+            bool in_band[kChunkBatch], valid[kChunkBatch];
+#pragma unroll
+            for (int c = 0; c < kChunkBatch; ++c) {
+                const int r = (b0 + c) * (64 / CPR) + lane_r;
+                const int m = m0 + wm * WTM + i * 32 + r;
+                const int n = n0 + wn * WTN + lane_cc * 8;
+                valid[c] = EVEN || (m < g.M && n < g.N);
+                in_band[c] = valid[c] && m >= band_lo && m < band_hi;
+                off[c] = in_band[c] ? (int64_t)(m - band_lo) * g.N + n : (int64_t)m * g.N + n;
             }
+            // first group of peers: issued before the patch is read
+            u32x4 pv[kChunkBatch][kPeerGroup];
+#pragma unroll
+            for (int c = 0; c < kChunkBatch; ++c)
+#pragma unroll
+                for (int q = 0; q < kPeerGroup; ++q)
+                    if (in_band[c] && q < g.n_peers)
+                        pv[c][q] = ld_stream((const u32x4*)(g.peers + q * g.peers_stride + off[c]));
+#pragma unroll
+            for (int c = 0; c < kChunkBatch; ++c) {
+                const int r = (b0 + c) * (64 / CPR) + lane_r;
+                const f32x4 lo = *(const f32x4*)(patch + r * EP_LD + lane_cc * 8);
+                const f32x4 hi = *(const f32x4*)(patch + r * EP_LD + lane_cc * 8 + 4);
+                f[c][0] = lo.x; f[c][1] = lo.y; f[c][2] = lo.z; f[c][3] = lo.w;
+                f[c][4] = hi.x; f[c][5] = hi.y; f[c][6] = hi.z; f[c][7] = hi.w;
+            }
+#pragma unroll
+            for (int c = 0; c < kChunkBatch; ++c)
+#pragma unroll
+                for (int q = 0; q < kPeerGroup; ++q)
+                    if (in_band[c] && q < g.n_peers) add8(pv[c][q], f[c]);
+            // second group (9..15 peers; KR_MAX_WORLD = 16), same pattern
+            if (g.n_peers > kPeerGroup) {
+#pragma unroll
+                for (int c = 0; c < kChunkBatch; ++c)
+#pragma unroll
+                    for (int q = 0; q < kPeerGroup; ++q)
+                        if (in_band[c] && kPeerGroup + q < g.n_peers)
+                            pv[c][q] = ld_stream(
+                                (const u32x4*)(g.peers + (kPeerGroup + q) * g.peers_stride + off[c]));
+#pragma unroll
+                for (int c = 0; c < kChunkBatch; ++c)
+#pragma unroll
+                    for (int q = 0; q < kPeerGroup; ++q)
+                        if (in_band[c] && kPeerGroup + q < g.n_peers) add8(pv[c][q], f[c]);
+            }
+#pragma unroll
+            for (int c = 0; c < kChunkBatch; ++c) {
+                if (in_band[c]) {
+                    const int n = n0 + wn * WTN + lane_cc * 8;
+                    if (g.bias != nullptr) add8(*(const u32x4*)(g.bias + n), f[c]);
+                    if (g.out_is_fp32) {
+                        float* o = (float*)g.out + off[c];
+                        *(f32x4*)o = f32x4{f[c][0], f[c][1], f[c][2], f[c][3]};
+                        *(f32x4*)(o + 4) = f32x4{f[c][4], f[c][5], f[c][6], f[c][7]};
+                    } else {
+                        st_stream((u32x4*)((uint16_t*)g.out + off[c]), pack8(f[c]));
+                    }
+                } else if (valid[c] && g.c_full != nullptr) {
+                    st_stream((u32x4*)(g.c_full + off[c]), pack8(f[c]));
+                }
+            }
+            __builtin_amdgcn_sched_barrier(0);
         }
-        __syncthreads();
     }
 }
 
@@ -426,10 +490,17 @@ static hipError_t launch_gemm(const GemmArgs& g, bool b_nt, bool even, hipStream
         }                                                                                             \
         hipLaunchKernelGGL(kfn, grid, block, LDS, st, g);                                             \
     } while (0)
-    if (b_nt) {
-        if (even) KR_LAUNCH(true, true); else KR_LAUNCH(true, false);
+    // The 256x256 tile is only instantiated for shapes it divides (its edge-handling variant
+    // would not fit the register file next to 256 accumulators).
+    if constexpr (BM >= 256) {
+        if (!even) return hipErrorInvalidValue;
+        if (b_nt) KR_LAUNCH(true, true); else KR_LAUNCH(false, true);
     } else {
-        if (even) KR_LAUNCH(false, true); else KR_LAUNCH(false, false);
+        if (b_nt) {
+            if (even) KR_LAUNCH(true, true); else KR_LAUNCH(true, false);
+        } else {
+            if (even) KR_LAUNCH(false, true); else KR_LAUNCH(false, false);
+        }
     }
 #undef KR_LAUNCH
     return hipGetLastError();
@@ -489,7 +560,7 @@ extern "C" int kr_gemm_reduce_bf16(const void* A, int64_t lda_m, int64_t lda_k, 
     // KRAKEN_AMD_GEMM_TILE=128|256 overrides the choice (testing and tuning)
     if (const char* t = getenv("KRAKEN_AMD_GEMM_TILE")) {
         if (t[0] == '1') big = false;
-        if (t[0] == '2') big = true;
+        if (t[0] == '2') big = (M % 256 == 0 && N % 256 == 0 && K % BK == 0);
     }
     const int bm = big ? 256 : 128, bn = big ? 256 : 128;
     g.tiles_m = (int)((M + bm - 1) / bm);

@@ -47,6 +47,7 @@ def gemm_reduce_scatter(a: torch.Tensor, b: torch.Tensor, **kwargs) -> torch.Ten
     else:
         assert c_scratch.dtype == torch.bfloat16 and tuple(c_scratch.shape) == (M, N) and c_scratch.is_contiguous()
     out = torch.empty((m_scatter, N), dtype=in_dtype, device=a.device)
+    # tile order rotated so that the band's tiles (the ones with extra epilogue traffic) run first
     _gemm.launch("gemm_reduce_scatter", a, b, M, N, peers, P, pstride, None,
-                 rank * m_scatter, m_scatter, c_scratch, out, 0)
+                 rank * m_scatter, m_scatter, c_scratch, out, rank * m_scatter)
     return out
