@@ -389,55 +389,59 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_reduce_kernel(const GemmArgs
     const int band_lo = g.band_row0, band_hi = g.band_row0 + g.band_rows;
     const int lane_r = lane / CPR, lane_cc = lane % CPR;   // chunk (it*64 + lane): row it*(64/CPR) + lane_r
 
+    // One batch of kChunkBatch chunks of the current slab.  NP >= 0: every row of the slab lies
+    // in the band and there are exactly NP peers (straight-line code, no per-lane branches);
+    // NP == -1: generic per-lane handling (band edge inside the slab, ragged tile, any peer
+    // count); NP == -2: no row of the slab lies in the band.
+    auto slab_batch = [&](auto np_c, int slab_m0, int b0) {
+        constexpr int NP = decltype(np_c)::value;
+        float f[kChunkBatch][8];
+        int64_t off[kChunkBatch];
+        bool in_band[kChunkBatch], valid[kChunkBatch];
+        const int n = n0 + wn * WTN + lane_cc * 8;
 #pragma unroll
-    for (int i = 0; i < TM; ++i) {
-        // MFMA layout: lane holds column (lane & 31); register v is row 8*(v/4) + 4*(lane>>5) + v%4
+        for (int c = 0; c < kChunkBatch; ++c) {
+            const int m = slab_m0 + (b0 + c) * (64 / CPR) + lane_r;
+            valid[c] = EVEN || (m < g.M && n < g.N);
+            in_band[c] = NP >= 0 ? true : NP == -2 ? false : (valid[c] && m >= band_lo && m < band_hi);
+            off[c] = in_band[c] ? (int64_t)(m - band_lo) * g.N + n : (int64_t)m * g.N + n;
+        }
+        constexpr int NG = NP >= 0 ? NP : kPeerGroup;   // peers fetched in the first group
+        u32x4 pv[kChunkBatch][NG > 0 ? NG : 1];
+        if constexpr (NP > 0) {
 #pragma unroll
-        for (int j = 0; j < TN; ++j)
+            for (int c = 0; c < kChunkBatch; ++c)
 #pragma unroll
-            for (int v = 0; v < 16; ++v) {
-                const int r = 8 * (v >> 2) + 4 * (lane >> 5) + (v & 3);
-                patch[r * EP_LD + j * 32 + (lane & 31)] = acc[i][j][v];
-            }
-        // keep the scheduler from pulling the accumulator reads of later slabs (256 registers
-        // in all) ahead of this point
-        __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-        for (int b0 = 0; b0 < EP_ITERS; b0 += kChunkBatch) {
-            float f[kChunkBatch][8];
-            int64_t off[kChunkBatch];
-            bool in_band[kChunkBatch], valid[kChunkBatch];
-#pragma unroll
-            for (int c = 0; c < kChunkBatch; ++c) {
-                const int r = (b0 + c) * (64 / CPR) + lane_r;
-                const int m = m0 + wm * WTM + i * 32 + r;
-                const int n = n0 + wn * WTN + lane_cc * 8;
-                valid[c] = EVEN || (m < g.M && n < g.N);
-                in_band[c] = valid[c] && m >= band_lo && m < band_hi;
-                off[c] = in_band[c] ? (int64_t)(m - band_lo) * g.N + n : (int64_t)m * g.N + n;
-            }
-            // first group of peers: issued before the patch is read
-            u32x4 pv[kChunkBatch][kPeerGroup];
+                for (int q = 0; q < NP; ++q)
+                    pv[c][q] = ld_stream((const u32x4*)(g.peers + q * g.peers_stride + off[c]));
+        } else if constexpr (NP == -1) {
 #pragma unroll
             for (int c = 0; c < kChunkBatch; ++c)
 #pragma unroll
                 for (int q = 0; q < kPeerGroup; ++q)
                     if (in_band[c] && q < g.n_peers)
                         pv[c][q] = ld_stream((const u32x4*)(g.peers + q * g.peers_stride + off[c]));
+        }
 #pragma unroll
-            for (int c = 0; c < kChunkBatch; ++c) {
-                const int r = (b0 + c) * (64 / CPR) + lane_r;
-                const f32x4 lo = *(const f32x4*)(patch + r * EP_LD + lane_cc * 8);
-                const f32x4 hi = *(const f32x4*)(patch + r * EP_LD + lane_cc * 8 + 4);
-                f[c][0] = lo.x; f[c][1] = lo.y; f[c][2] = lo.z; f[c][3] = lo.w;
-                f[c][4] = hi.x; f[c][5] = hi.y; f[c][6] = hi.z; f[c][7] = hi.w;
-            }
+        for (int c = 0; c < kChunkBatch; ++c) {
+            const int r = (b0 + c) * (64 / CPR) + lane_r;
+            const f32x4 lo = *(const f32x4*)(patch + r * EP_LD + lane_cc * 8);
+            const f32x4 hi = *(const f32x4*)(patch + r * EP_LD + lane_cc * 8 + 4);
+            f[c][0] = lo.x; f[c][1] = lo.y; f[c][2] = lo.z; f[c][3] = lo.w;
+            f[c][4] = hi.x; f[c][5] = hi.y; f[c][6] = hi.z; f[c][7] = hi.w;
+        }
+        if constexpr (NP > 0) {
+#pragma unroll
+            for (int c = 0; c < kChunkBatch; ++c)
+#pragma unroll
+                for (int q = 0; q < NP; ++q) add8(pv[c][q], f[c]);
+        } else if constexpr (NP == -1) {
 #pragma unroll
             for (int c = 0; c < kChunkBatch; ++c)
 #pragma unroll
                 for (int q = 0; q < kPeerGroup; ++q)
                     if (in_band[c] && q < g.n_peers) add8(pv[c][q], f[c]);
-            // second group (9..15 peers; KR_MAX_WORLD = 16), same pattern
+            // second group (9..15 peers), same pattern
             if (g.n_peers > kPeerGroup) {
 #pragma unroll
                 for (int c = 0; c < kChunkBatch; ++c)
@@ -452,21 +456,67 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_reduce_kernel(const GemmArgs
                     for (int q = 0; q < kPeerGroup; ++q)
                         if (in_band[c] && kPeerGroup + q < g.n_peers) add8(pv[c][q], f[c]);
             }
+        }
+        if constexpr (NP != -2) {
+            if (g.bias != nullptr) {
+                const u32x4 bv = *(const u32x4*)(g.bias + (EVEN ? n : min(n, g.N - 8)));
 #pragma unroll
-            for (int c = 0; c < kChunkBatch; ++c) {
-                if (in_band[c]) {
-                    const int n = n0 + wn * WTN + lane_cc * 8;
-                    if (g.bias != nullptr) add8(*(const u32x4*)(g.bias + n), f[c]);
-                    if (g.out_is_fp32) {
-                        float* o = (float*)g.out + off[c];
-                        *(f32x4*)o = f32x4{f[c][0], f[c][1], f[c][2], f[c][3]};
-                        *(f32x4*)(o + 4) = f32x4{f[c][4], f[c][5], f[c][6], f[c][7]};
-                    } else {
-                        st_stream((u32x4*)((uint16_t*)g.out + off[c]), pack8(f[c]));
-                    }
-                } else if (valid[c] && g.c_full != nullptr) {
-                    st_stream((u32x4*)(g.c_full + off[c]), pack8(f[c]));
+                for (int c = 0; c < kChunkBatch; ++c)
+                    if (in_band[c]) add8(bv, f[c]);
+            }
+        }
+#pragma unroll
+        for (int c = 0; c < kChunkBatch; ++c) {
+            if (in_band[c]) {
+                if (g.out_is_fp32) {
+                    float* o = (float*)g.out + off[c];
+                    *(f32x4*)o = f32x4{f[c][0], f[c][1], f[c][2], f[c][3]};
+                    *(f32x4*)(o + 4) = f32x4{f[c][4], f[c][5], f[c][6], f[c][7]};
+                } else {
+                    st_stream((u32x4*)((uint16_t*)g.out + off[c]), pack8(f[c]));
                 }
+            } else if (valid[c] && g.c_full != nullptr) {
+                st_stream((u32x4*)(g.c_full + off[c]), pack8(f[c]));
+            }
+        }
+    };
+
+    // the wave's first row, as a scalar: the slab classification below must branch uniformly
+    const int wave_m0 = __builtin_amdgcn_readfirstlane(m0 + wm * WTM);
+    // The slab loop is a real loop (its body, with the specialised batch variants, exists
+    // once); only the copy of slab i's accumulators to the patch is selected by a uniform
+    // if-chain, because accumulator registers can only be indexed statically.
+#pragma nounroll
+    for (int i = 0; i < TM; ++i) {
+        // MFMA layout: lane holds column (lane & 31); register v is row 8*(v/4) + 4*(lane>>5) + v%4
+#pragma unroll
+        for (int ii = 0; ii < TM; ++ii) {
+            if (i == ii) {
+#pragma unroll
+                for (int j = 0; j < TN; ++j)
+#pragma unroll
+                    for (int v = 0; v < 16; ++v) {
+                        const int r = 8 * (v >> 2) + 4 * (lane >> 5) + (v & 3);
+                        patch[r * EP_LD + j * 32 + (lane & 31)] = acc[ii][j][v];
+                    }
+            }
+        }
+        // keep the scheduler from pulling the accumulator reads of later slabs (256 registers
+        // in all) ahead of this point
+        __builtin_amdgcn_sched_barrier(0);
+        const int slab_m0 = wave_m0 + i * 32;
+        const bool all_in = EVEN && slab_m0 >= band_lo && slab_m0 + 32 <= band_hi;
+        const bool all_out = EVEN && (slab_m0 + 32 <= band_lo || slab_m0 >= band_hi);
+#pragma unroll
+        for (int b0 = 0; b0 < EP_ITERS; b0 += kChunkBatch) {
+            if (all_out) {
+                slab_batch(std::integral_constant<int, -2>{}, slab_m0, b0);
+            } else if (all_in && g.n_peers == 7) {
+                slab_batch(std::integral_constant<int, 7>{}, slab_m0, b0);
+            } else if (all_in && g.n_peers == 0) {
+                slab_batch(std::integral_constant<int, 0>{}, slab_m0, b0);
+            } else {
+                slab_batch(std::integral_constant<int, -1>{}, slab_m0, b0);
             }
             __builtin_amdgcn_sched_barrier(0);
         }
