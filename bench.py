@@ -557,9 +557,11 @@ def main() -> None:
                 continue
             wl = ctor()
             big_gemm = wl.bound == "mfma" or wl.flops
-            steps = max(10, args.steps // 10) if big_gemm else args.steps
+            # GEMM steps take ~0.4 ms: half as many timed steps, but a longer warm-up -- the
+            # matrix-core clocks need some tens of milliseconds of load to settle
+            steps = max(10, args.steps // 2) if big_gemm else args.steps
             try:
-                r = measure(wl, steps, min(args.warmup, 5) if big_gemm else args.warmup, dev, not args.no_cpu, 6.0)
+                r = measure(wl, steps, max(args.warmup, 60) if big_gemm else args.warmup, dev, not args.no_cpu, 6.0)
                 r["steps"] = steps
             except Exception as e:  # a failing side workload must not hide the headline number
                 r = {"workload": wl.name, "error": f"{type(e).__name__}: {e}"}

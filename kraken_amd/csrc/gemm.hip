@@ -69,6 +69,14 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_reduce_kernel(const GemmArgs
     tile_schedule(g, tile_m, tile_n);
     const int m0 = tile_m * BM, n0 = tile_n * BN;
 
+    f32x16 acc[TM][TN];
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
+
     // ---- operand staging: global -> registers -> LDS, one 16-byte chunk per "unit" ------
     // Global loads are buffer loads: a wave-uniform resource descriptor (tile base), a
     // per-thread 32-bit byte offset that never changes, and a wave-uniform scalar offset that
@@ -192,14 +200,6 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_reduce_kernel(const GemmArgs
         if (q < TM) af[buf][q] = *(lds_frag)(size_t)(fa_off[q] ^ (uint32_t)(ks << 5) ^ other);
         else bfr[buf][q - TM] = *(lds_frag)(size_t)(fb_off[q - TM] ^ (uint32_t)(ks << 5) ^ other);
     };
-
-    f32x16 acc[TM][TN];
-#pragma unroll
-    for (int i = 0; i < TM; ++i)
-#pragma unroll
-        for (int j = 0; j < TN; ++j)
-#pragma unroll
-            for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
 
     // ---- software pipeline ---------------------------------------------------------------
     // Iteration t computes tile t from LDS stage t&1 while (a) the registers holding tile
@@ -421,7 +421,7 @@ extern "C" int kr_gemm_reduce_bf16(const void* A, int64_t lda_m, int64_t lda_k, 
     // work per LDS/HBM byte; it needs enough tiles to fill 256 CUs and a K loop
     // long enough to amortise its epilogue.  Otherwise 128x128 tiles, several
     // of which share a CU so that one tile's epilogue overlaps another's MFMAs.
-    bool big = (M % 256 == 0 && N % 256 == 0 && K % BK == 0 && (M / 256) * (N / 256) >= 256 && K >= 2048);
+    bool big = (M % 256 == 0 && N % 256 == 0 && K % BK == 0 && (M / 256) * (N / 256) >= 256 && K >= 256);
     // KRAKEN_AMD_GEMM_TILE=128|256 overrides the choice (testing and tuning)
     if (const char* t = getenv("KRAKEN_AMD_GEMM_TILE")) {
         if (t[0] == '1') big = false;
