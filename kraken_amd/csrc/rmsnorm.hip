@@ -6,6 +6,8 @@
 // of squares is reduced inside each wavefront with DPP lane permutes, then
 // across the wavefronts of the workgroup through a few words of LDS that every
 // thread re-reads in the same order, so all threads hold the same rstd.
+#include <stdlib.h>
+
 #include "common.h"
 
 namespace kr {
@@ -29,11 +31,16 @@ __global__ __launch_bounds__(kMaxThreads) void reduce_rmsnorm_kernel(
     float s[VPT][8];
     u32x4 wv[VPT];
 
-    // issue the weight loads early; they are shared by all rows and stay in L2
+    // issue the weight loads early (they are shared by all rows and stay in L2); rows long
+    // enough to need 4+ vectors per thread fetch them after the reduction instead, to stay
+    // inside the 128 registers a 1024-thread workgroup leaves per thread
+    constexpr bool kEarlyWeights = VPT < 4;
+    if (kEarlyWeights) {
 #pragma unroll
-    for (int v = 0; v < VPT; ++v) {
-        const int c = tid + v * nthr;
-        wv[v] = c < d_vec ? wgt[c] : u32x4{0, 0, 0, 0};
+        for (int v = 0; v < VPT; ++v) {
+            const int c = tid + v * nthr;
+            wv[v] = c < d_vec ? wgt[c] : u32x4{0, 0, 0, 0};
+        }
     }
 
 #pragma unroll
@@ -48,7 +55,7 @@ __global__ __launch_bounds__(kMaxThreads) void reduce_rmsnorm_kernel(
         }
     }
 
-    if constexpr (WT > 0 && WT * VPT <= 16) {
+    if constexpr (WT > 0 && WT * VPT <= 16 && VPT < 4) {
         // all W*VPT loads of the thread in flight before the first add
         u32x4 x[WT][VPT];
 #pragma unroll
@@ -63,16 +70,24 @@ __global__ __launch_bounds__(kMaxThreads) void reduce_rmsnorm_kernel(
 #pragma unroll
             for (int v = 0; v < VPT; ++v) add8(x[r][v], s[v]);
     } else {
-        // long rows: one slice at a time keeps the register count bounded
-        for (int r = 0; r < W; ++r) {
-            u32x4 x[VPT];
+        // long rows (or run-time W): G slices at a time, G * VPT <= 16 loads in flight per thread
+        constexpr int G = VPT >= 4 ? 8 / VPT : 16 / VPT;   // long rows keep 64 row registers: fewer loads in flight
+#pragma unroll 1
+        for (int r0 = 0; r0 < W; r0 += G) {
+            u32x4 x[G][VPT];
 #pragma unroll
-            for (int v = 0; v < VPT; ++v) {
-                const int c = tid + v * nthr;
-                x[v] = c < d_vec ? ld_stream(stack + r * slice_stride_v + row_v + c) : u32x4{0, 0, 0, 0};
-            }
+            for (int gi = 0; gi < G; ++gi)
 #pragma unroll
-            for (int v = 0; v < VPT; ++v) add8(x[v], s[v]);
+                for (int v = 0; v < VPT; ++v) {
+                    const int c = tid + v * nthr;
+                    x[gi][v] = (r0 + gi < W && c < d_vec)
+                                   ? ld_stream(stack + (r0 + gi) * slice_stride_v + row_v + c)
+                                   : u32x4{0, 0, 0, 0};
+                }
+#pragma unroll
+            for (int gi = 0; gi < G; ++gi)
+#pragma unroll
+                for (int v = 0; v < VPT; ++v) add8(x[gi][v], s[v]);
         }
     }
 
@@ -98,7 +113,7 @@ __global__ __launch_bounds__(kMaxThreads) void reduce_rmsnorm_kernel(
         const int c = tid + v * nthr;
         if (c < d_vec) {
             float wf[8], o[8];
-            unpack8(wv[v], wf);
+            unpack8(kEarlyWeights ? wv[v] : wgt[c], wf);
 #pragma unroll
             for (int j = 0; j < 8; ++j) o[j] = (s[v][j] * rstd) * wf[j];
             st_stream(y + row_v + c, pack8(o));
@@ -145,9 +160,14 @@ static hipError_t launch_row1(int W, int mode, dim3 grid, dim3 block, hipStream_
 static void row_geometry(int d_vec, int* threads, int* vpt) {
     int v = 1;
     while ((int64_t)v * kMaxThreads < d_vec) v *= 2;           // 1,2,4,8
-    // prefer 2 vectors per thread once a row spans more than 256 vectors: fewer
-    // wavefronts to synchronise, same bytes in flight per CU
-    if (v == 1 && d_vec > 256) v = 2;
+    // (one vector per thread measured best: 78 % of HBM peak at D = 4096/8192 against 75-77 %
+    // with two; more wavefronts per row cost less than fewer loads in flight per thread)
+    // KRAKEN_AMD_ROW_VPT=1|2|4|8 overrides the vectors per thread (tuning); ignored if a row
+    // would need more than 1024 threads
+    if (const char* e = getenv("KRAKEN_AMD_ROW_VPT")) {
+        const int o = atoi(e);
+        if ((o == 1 || o == 2 || o == 4 || o == 8) && (int64_t)o * kMaxThreads >= d_vec) v = o;
+    }
     int t = (d_vec + v - 1) / v;
     t = (t + kWave - 1) / kWave * kWave;
     *threads = t;
