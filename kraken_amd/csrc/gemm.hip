@@ -14,9 +14,11 @@
 // Row-major B ([K,N], N contiguous) is transposed on its way into LDS: a
 // thread loads an 8(k) x 8(n) block with eight 128-bit loads, transposes it in
 // registers with byte permutes and writes eight 128-bit [n][8 k] chunks.
-// Epilogue: accumulators go through a per-wave LDS patch to turn the MFMA
-// layout into row-contiguous 8-element vectors, so peers, bias and output are
-// all moved with 128-bit accesses covering whole 256-byte row segments.
+// Epilogue (shared with the LDS-DMA kernel for 256x256 tiles): accumulators go
+// through a per-wave LDS patch to turn the MFMA layout into row-contiguous
+// 8-element vectors, so peers, bias and output are all moved with 128-bit
+// accesses covering whole row segments.  This file also holds the C entry point
+// and the choice between the two kernels.
 #include <stdlib.h>
 
 #include <type_traits>
@@ -54,8 +56,7 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_reduce_kernel(const GemmArgs
     static_assert(BM % (WM * 32) == 0 && BN % (WN * 32) == 0, "wave tile must be a multiple of 32");
     static_assert((BM * 8) % T == 0 && (BN * 8) % T == 0 && (BN % T == 0 || BN < T), "load split");
     // epilogue patch: 32 rows x WTN fp32 per wave, rows padded by 4 floats
-    constexpr int EP_LD = WTN + 4;
-    constexpr int EP_WAVE = 32 * EP_LD * 4;
+    constexpr int EP_WAVE = 32 * (WTN + 4) * 4;
     static_assert(EP_WAVE * WM * WN <= 2 * STAGE, "epilogue patch must fit in the pipeline LDS");
 
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
@@ -224,9 +225,6 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_reduce_kernel(const GemmArgs
     uint32_t nxt = STAGE;   // stage (relative to stage 0) that receives tile t+1
     static_assert((STAGE & (STAGE - 1)) == 0, "stage selection by XOR needs a power-of-two stage size");
     auto staging_job = [&](int rs, int j, int k2) {
-#ifdef KR_EXP_NOSTAGING
-        return;
-#endif
         if (j < A_ITERS) {
             store_a_unit(rs, j, nxt);
             load_a_unit(rs, j, k2);
@@ -249,7 +247,7 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_reduce_kernel(const GemmArgs
 #pragma unroll
         for (int s = 0; s < NM; ++s) {
             const int i = s / TN, j = s % TN;
-            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[buf][i], bfr[buf][j], acc[i][j], 0, 0, 0);
+            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bfr[buf][j], af[buf][i], acc[i][j], 0, 0, 0);
 #pragma unroll
             for (int q = s * NF / NM; q < (s + 1) * NF / NM; ++q)
                 read_frag(q, (ks + 1) & 3, ks == 3 ? STAGE : 0, buf ^ 1);
@@ -282,9 +280,7 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_reduce_kernel(const GemmArgs
         mfma_step(std::integral_constant<int, 2>{}, rs_c, k2);
         // every LDS access of this wave so far has completed; then all waves meet
         __builtin_amdgcn_s_waitcnt(0xc07f);   // lgkmcnt(0) only: the global loads stay in flight
-#ifndef KR_EXP_NOBARRIER
         __builtin_amdgcn_s_barrier();
-#endif
         KR_SCHED_FENCE();
         // sub-step 3 reads the fragments of sub-step 0 of tile t+1
         mfma_step(std::integral_constant<int, 3>{}, rs_c, k2);
@@ -335,7 +331,7 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_reduce_kernel(const GemmArgs
     // LDS is reused by the epilogue
     __syncthreads();
 
-    gemm_epilogue<BM, WTM, WTN, TM, TN, EVEN, EP_LD, EP_WAVE>(g, acc, smem, m0, n0, wm, wn, lane, wave);
+    gemm_epilogue<BM, WTM, WTN, TM, TN, EVEN, EP_WAVE>(g, acc, smem, m0, n0, wm, wn, lane, wave);
 }
 
 template <int BM, int BN, int WM, int WN>
@@ -355,17 +351,10 @@ static hipError_t launch_gemm(const GemmArgs& g, bool b_nt, bool even, hipStream
         }                                                                                             \
         hipLaunchKernelGGL(kfn, grid, block, LDS, st, g);                                             \
     } while (0)
-    // The 256x256 tile is only instantiated for shapes it divides (its edge-handling variant
-    // would not fit the register file next to 256 accumulators).
-    if constexpr (BM >= 256) {
-        if (!even) return hipErrorInvalidValue;
-        if (b_nt) KR_LAUNCH(true, true); else KR_LAUNCH(false, true);
+    if (b_nt) {
+        if (even) KR_LAUNCH(true, true); else KR_LAUNCH(true, false);
     } else {
-        if (b_nt) {
-            if (even) KR_LAUNCH(true, true); else KR_LAUNCH(true, false);
-        } else {
-            if (even) KR_LAUNCH(false, true); else KR_LAUNCH(false, false);
-        }
+        if (even) KR_LAUNCH(false, true); else KR_LAUNCH(false, false);
     }
 #undef KR_LAUNCH
     return hipGetLastError();
@@ -417,31 +406,25 @@ extern "C" int kr_gemm_reduce_bf16(const void* A, int64_t lda_m, int64_t lda_k, 
     g.out = out;
     g.out_is_fp32 = out_is_fp32;
 
-    // Tile choice: the 256x256 tile (4 waves x 128x128) has the highest MFMA
-    // work per LDS/HBM byte; it needs enough tiles to fill 256 CUs and a K loop
-    // long enough to amortise its epilogue.  Otherwise 128x128 tiles, several
-    // of which share a CU so that one tile's epilogue overlaps another's MFMAs.
-    bool big = (M % 256 == 0 && N % 256 == 0 && K % BK == 0 && (M / 256) * (N / 256) >= 256 && K >= 256);
+    // Tile choice: the 256x256 tile of the LDS-DMA kernel (4 waves x 128x128) has the highest
+    // MFMA work per LDS/HBM byte; it needs a shape it divides, enough tiles to fill 256 CUs and
+    // a K loop long enough to amortise its epilogue.  Otherwise 128x128 tiles, two of which
+    // share a CU so that one tile's epilogue overlaps the other's MFMAs.
+    bool big = (M / 256) * (N / 256) >= 256 && K >= 256;
     // KRAKEN_AMD_GEMM_TILE=128|256 overrides the choice (testing and tuning)
     if (const char* t = getenv("KRAKEN_AMD_GEMM_TILE")) {
         if (t[0] == '1') big = false;
-        if (t[0] == '2') big = (M % 256 == 0 && N % 256 == 0 && K % BK == 0);
+        if (t[0] == '2') big = true;
     }
-    const int bm = big ? 256 : 128, bn = big ? 256 : 128;
+    const bool dtl = big && gemm_dtl_supported(g);
+    const int bm = dtl ? 256 : 128, bn = bm;
     g.tiles_m = (int)((M + bm - 1) / bm);
     g.tiles_n = (int)((N + bn - 1) / bn);
     if ((int64_t)g.tiles_m * g.tiles_n > 0x7fffffffLL) return KR_ERR_BAD_DIM;
     int64_t pt = tile_pivot / bm;
     g.pivot_tiles = (int)(((pt % g.tiles_m) + g.tiles_m) % g.tiles_m);
     const bool even = (M % bm == 0 && N % bn == 0 && K % BK == 0);
-    // KRAKEN_AMD_GEMM_PATH=staged keeps the register-staged main loop for the 256x256 tile
-    // (testing and tuning); the default for shapes it divides is the LDS-DMA kernel.
-    bool dtl = big && gemm_dtl_supported(g);
-    if (const char* t = getenv("KRAKEN_AMD_GEMM_PATH")) {
-        if (t[0] == 's') dtl = false;
-    }
-    hipError_t e = dtl   ? launch_gemm_dtl(g, b_nt, (hipStream_t)stream)
-                   : big ? launch_gemm<256, 256, 2, 2>(g, b_nt, even, (hipStream_t)stream)
-                         : launch_gemm<128, 128, 2, 2>(g, b_nt, even, (hipStream_t)stream);
+    hipError_t e = dtl ? launch_gemm_dtl(g, b_nt, (hipStream_t)stream)
+                       : launch_gemm<128, 128, 2, 2>(g, b_nt, even, (hipStream_t)stream);
     return (int)e;
 }

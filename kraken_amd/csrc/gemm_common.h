@@ -58,143 +58,246 @@ __device__ __forceinline__ void tile_schedule(const GemmArgs& g, int& tile_m_out
     tile_n_out = tile_n;
 }
 
-// Fused epilogue of one workgroup tile.  `acc` are the 32x32 MFMA accumulators of this wave
-// (TM x TN blocks), `smem` the workgroup's LDS (free for reuse: every wave has passed a
-// barrier after its last read of the operand stages).
-template <int BM, int WTM, int WTN, int TM, int TN, bool EVEN, int EP_LD, int EP_WAVE>
-__device__ __forceinline__ void gemm_epilogue(const GemmArgs& g, const f32x16 (&acc)[TM][TN], unsigned char* smem,
-                                              int m0, int n0, int wm, int wn, int lane, int wave) {
+// Fused epilogue of one workgroup tile.  `acc` are this wave's 32x32 MFMA accumulators (TM x TN
+// blocks) in the TRANSPOSED layout the kernels produce by passing the B fragment as the first
+// MFMA operand: lane holds row (lane & 31) of the block, register v is column
+// 8*(v/4) + 4*(lane>>5) + v%4 -- four consecutive columns per register quad, so a quad is one
+// contiguous store into a row-major LDS patch.  `smem` is the workgroup's LDS (free for reuse:
+// every wave has passed a barrier after its last read of the operand stages).
+//
+// F32 = false (bf16 result): the product is rounded to bf16 on its way into the patch, exactly
+// as the reference rounds a rank's partial product before it is summed
+// (kraken/fused/gemm_one_shot_all_reduce_fused.py:120-135); partial sums of the peers and the
+// bias are then added in fp32 in the order own, peer 0, 1, ..., bias.
+// F32 = true (fp32 result, used by the split-fp32 emulation): the patch holds fp32.
+template <bool F32, int BM, int WTM, int WTN, int TM, int TN, bool EVEN, int EP_WAVE>
+__device__ __forceinline__ void gemm_epilogue_impl(const GemmArgs& g, const f32x16 (&acc)[TM][TN], unsigned char* smem,
+                                                   int m0, int n0, int wm, int wn, int lane, int wave) {
     // After the barrier above no wave reads the pipeline stages any more, and from here on
     // every wave touches only its own LDS patch, so no further workgroup barrier is needed
     // (LDS requests of one wave are served in order).  Per 32-row slab the accumulators are
-    // written to the patch in MFMA layout and read back as row-contiguous 8-element chunks.
-    // The partial sums of the other ranks are fetched kPeerGroup peers x kChunkBatch chunks at
-    // a time, all loads issued before the first add, so a band tile keeps dozens of 1 KiB
-    // wave-loads in flight instead of waiting for one HBM round trip per peer.
-    float* patch = (float*)(smem + wave * EP_WAVE);
+    // written to the patch and read back as row-contiguous 8-element chunks.
+    //
+    // Loads and stores share one in-order counter on this hardware: waiting for a load that
+    // was issued after a store also waits until that store has been acknowledged by memory,
+    // a round trip of thousands of cycles.  So nothing in the store path may depend on a
+    // load issued behind a store: the bias is fetched once, before the first store, and the
+    // partial sums of the other ranks are fetched one batch ahead (the loads of batch b+1 are
+    // issued before the stores of batch b), so every wait leaves the younger stores pending.
+    typedef typename std::conditional<F32, float, uint16_t>::type patch_t;
+    // row pitch in elements: 16 bytes of padding keep the quad stores of 16 (bf16: 8-byte) or
+    // 8 (fp32: 16-byte) lanes on distinct banks and the rows 16-byte aligned
+    constexpr int LD = WTN + (F32 ? 4 : 8);
+    static_assert(32 * LD * (int)sizeof(patch_t) <= EP_WAVE, "patch exceeds the wave's share of LDS");
+    patch_t* patch = (patch_t*)(smem + wave * EP_WAVE);
     constexpr int CPR = WTN / 8;            // 8-element chunks per patch row
     constexpr int EP_ITERS = 32 * CPR / 64; // chunks per lane per 32-row slab
     constexpr int kChunkBatch = BM >= 256 ? 4 : 2;   // the small tile keeps its register count low (occupancy)
-    constexpr int kPeerGroup = 8;
-    static_assert(2 * kPeerGroup >= KR_MAX_WORLD - 1, "two peer groups must cover every world size");
+    constexpr int kPeerGroup = 4;           // peers fetched together by the generic path
     const int band_lo = g.band_row0, band_hi = g.band_row0 + g.band_rows;
     const int lane_r = lane / CPR, lane_cc = lane % CPR;   // chunk (it*64 + lane): row it*(64/CPR) + lane_r
+    const int n = n0 + wn * WTN + lane_cc * 8;             // first of the lane's 8 columns, same for every chunk
 
-    // One batch of kChunkBatch chunks of the current slab.  NP >= 0: every row of the slab lies
-    // in the band and there are exactly NP peers (straight-line code, no per-lane branches);
-    // NP == -1: generic per-lane handling (band edge inside the slab, ragged tile, any peer
-    // count); NP == -2: no row of the slab lies in the band.
-    auto slab_batch = [&](auto np_c, int slab_m0, int b0) {
-        constexpr int NP = decltype(np_c)::value;
-        float f[kChunkBatch][8];
-        int64_t off[kChunkBatch];
-        bool in_band[kChunkBatch], valid[kChunkBatch];
-        const int n = n0 + wn * WTN + lane_cc * 8;
-#pragma unroll
-        for (int c = 0; c < kChunkBatch; ++c) {
-            const int m = slab_m0 + (b0 + c) * (64 / CPR) + lane_r;
-            valid[c] = EVEN || (m < g.M && n < g.N);
-            in_band[c] = NP >= 0 ? true : NP == -2 ? false : (valid[c] && m >= band_lo && m < band_hi);
-            off[c] = in_band[c] ? (int64_t)(m - band_lo) * g.N + n : (int64_t)m * g.N + n;
-        }
-        constexpr int NG = NP >= 0 ? NP : kPeerGroup;   // peers fetched in the first group
-        u32x4 pv[kChunkBatch][NG > 0 ? NG : 1];
-        if constexpr (NP > 0) {
-#pragma unroll
-            for (int c = 0; c < kChunkBatch; ++c)
-#pragma unroll
-                for (int q = 0; q < NP; ++q)
-                    pv[c][q] = ld_stream((const u32x4*)(g.peers + q * g.peers_stride + off[c]));
-        } else if constexpr (NP == -1) {
-#pragma unroll
-            for (int c = 0; c < kChunkBatch; ++c)
-#pragma unroll
-                for (int q = 0; q < kPeerGroup; ++q)
-                    if (in_band[c] && q < g.n_peers)
-                        pv[c][q] = ld_stream((const u32x4*)(g.peers + q * g.peers_stride + off[c]));
-        }
-#pragma unroll
-        for (int c = 0; c < kChunkBatch; ++c) {
-            const int r = (b0 + c) * (64 / CPR) + lane_r;
-            const f32x4 lo = *(const f32x4*)(patch + r * EP_LD + lane_cc * 8);
-            const f32x4 hi = *(const f32x4*)(patch + r * EP_LD + lane_cc * 8 + 4);
-            f[c][0] = lo.x; f[c][1] = lo.y; f[c][2] = lo.z; f[c][3] = lo.w;
-            f[c][4] = hi.x; f[c][5] = hi.y; f[c][6] = hi.z; f[c][7] = hi.w;
-        }
-        if constexpr (NP > 0) {
-#pragma unroll
-            for (int c = 0; c < kChunkBatch; ++c)
-#pragma unroll
-                for (int q = 0; q < NP; ++q) add8(pv[c][q], f[c]);
-        } else if constexpr (NP == -1) {
-#pragma unroll
-            for (int c = 0; c < kChunkBatch; ++c)
-#pragma unroll
-                for (int q = 0; q < kPeerGroup; ++q)
-                    if (in_band[c] && q < g.n_peers) add8(pv[c][q], f[c]);
-            // second group (9..15 peers), same pattern
-            if (g.n_peers > kPeerGroup) {
-#pragma unroll
-                for (int c = 0; c < kChunkBatch; ++c)
-#pragma unroll
-                    for (int q = 0; q < kPeerGroup; ++q)
-                        if (in_band[c] && kPeerGroup + q < g.n_peers)
-                            pv[c][q] = ld_stream(
-                                (const u32x4*)(g.peers + (kPeerGroup + q) * g.peers_stride + off[c]));
-#pragma unroll
-                for (int c = 0; c < kChunkBatch; ++c)
-#pragma unroll
-                    for (int q = 0; q < kPeerGroup; ++q)
-                        if (in_band[c] && kPeerGroup + q < g.n_peers) add8(pv[c][q], f[c]);
-            }
-        }
-        if constexpr (NP != -2) {
-            if (g.bias != nullptr) {
-                const u32x4 bv = *(const u32x4*)(g.bias + (EVEN ? n : min(n, g.N - 8)));
-#pragma unroll
-                for (int c = 0; c < kChunkBatch; ++c)
-                    if (in_band[c]) add8(bv, f[c]);
-            }
-        }
-#pragma unroll
-        for (int c = 0; c < kChunkBatch; ++c) {
-            if (in_band[c]) {
-                if (g.out_is_fp32) {
-                    float* o = (float*)g.out + off[c];
-                    *(f32x4*)o = f32x4{f[c][0], f[c][1], f[c][2], f[c][3]};
-                    *(f32x4*)(o + 4) = f32x4{f[c][4], f[c][5], f[c][6], f[c][7]};
-                } else {
-                    st_stream((u32x4*)((uint16_t*)g.out + off[c]), pack8(f[c]));
-                }
-            } else if (valid[c] && g.c_full != nullptr) {
-                st_stream((u32x4*)(g.c_full + off[c]), pack8(f[c]));
-            }
-        }
+    float bias_f[8];
+    zero8(bias_f);
+    const bool has_bias = g.bias != nullptr;
+    if (has_bias) add8(*(const u32x4*)(g.bias + (EVEN ? n : min(n, g.N - 8))), bias_f);
+
+    // Round-to-nearest-even pack of two fp32 to bf16, pinned where it is written: the
+    // accumulators do not change inside the slab loop, so an ordinary conversion would be
+    // hoisted out of it for all slabs at once, at the price of 128 more live registers.
+    auto pack_here = [](float lo, float hi) __attribute__((always_inline)) {
+        uint32_t r;
+        asm volatile("v_cvt_pk_bf16_f32 %0, %1, %2" : "=v"(r) : "v"(lo), "v"(hi));
+        return r;
     };
-
-    // the wave's first row, as a scalar: the slab classification below must branch uniformly
-    const int wave_m0 = __builtin_amdgcn_readfirstlane(m0 + wm * WTM);
-    // The slab loop is a real loop (its body, with the specialised batch variants, exists
-    // once); only the copy of slab i's accumulators to the patch is selected by a uniform
-    // if-chain, because accumulator registers can only be indexed statically.
-#pragma nounroll
-    for (int i = 0; i < TM; ++i) {
-        // MFMA layout: lane holds column (lane & 31); register v is row 8*(v/4) + 4*(lane>>5) + v%4
+    // copy of slab i's accumulators to the patch.  Accumulator registers can only be indexed
+    // statically, hence the uniform if-chain inside a rolled slab loop.
+    auto copy_slab = [&](int i) __attribute__((always_inline)) {
+        patch_t* row = patch + (lane & 31) * LD + 4 * (lane >> 5);
 #pragma unroll
         for (int ii = 0; ii < TM; ++ii) {
             if (i == ii) {
 #pragma unroll
                 for (int j = 0; j < TN; ++j)
 #pragma unroll
-                    for (int v = 0; v < 16; ++v) {
-                        const int r = 8 * (v >> 2) + 4 * (lane >> 5) + (v & 3);
-                        patch[r * EP_LD + j * 32 + (lane & 31)] = acc[ii][j][v];
+                    for (int q = 0; q < 4; ++q) {
+                        const f32x16& a = acc[ii][j];
+                        if constexpr (F32) {
+                            *(f32x4*)(row + j * 32 + 8 * q) = f32x4{a[4 * q], a[4 * q + 1], a[4 * q + 2], a[4 * q + 3]};
+                        } else {
+                            typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+                            *(u32x2*)(row + j * 32 + 8 * q) =
+                                u32x2{pack_here(a[4 * q], a[4 * q + 1]), pack_here(a[4 * q + 2], a[4 * q + 3])};
+                        }
                     }
+                // a distinct statement per case: identical case bodies would be merged into one
+                // with a run-time accumulator index, which forces the accumulators into memory
+                asm volatile("; accumulators of slab %0 copied" ::"n"(ii));
             }
         }
         // keep the scheduler from pulling the accumulator reads of later slabs (256 registers
         // in all) ahead of this point
         __builtin_amdgcn_sched_barrier(0);
+    };
+    // one chunk of the current slab: as stored (bf16 patch) or as fp32 values
+    auto read_raw = [&](int chunk) __attribute__((always_inline)) {
+        const int r = chunk * (64 / CPR) + lane_r;
+        return *(const u32x4*)(patch + r * LD + lane_cc * 8);
+    };
+    auto read_chunk = [&](int chunk, float (&f)[8]) __attribute__((always_inline)) {
+        if constexpr (F32) {
+            const int r = chunk * (64 / CPR) + lane_r;
+            const f32x4 lo = *(const f32x4*)(patch + r * LD + lane_cc * 8);
+            const f32x4 hi = *(const f32x4*)(patch + r * LD + lane_cc * 8 + 4);
+            f[0] = lo.x; f[1] = lo.y; f[2] = lo.z; f[3] = lo.w;
+            f[4] = hi.x; f[5] = hi.y; f[6] = hi.z; f[7] = hi.w;
+        } else {
+            unpack8(read_raw(chunk), f);
+        }
+    };
+    auto store_out = [&](int64_t off, const float (&f)[8]) __attribute__((always_inline)) {
+        if constexpr (F32) {
+            float* o = (float*)g.out + off;
+            *(f32x4*)o = f32x4{f[0], f[1], f[2], f[3]};
+            *(f32x4*)(o + 4) = f32x4{f[4], f[5], f[6], f[7]};
+        } else {
+            st_stream((u32x4*)((uint16_t*)g.out + off), pack8(f));
+        }
+    };
+
+    // the wave's first row, as a scalar: the classification below must branch uniformly
+    const int wave_m0 = __builtin_amdgcn_readfirstlane(m0 + wm * WTM);
+
+    // ---- every row of the wave lies in the band and there are exactly 7 peers ---------------
+    // (the eight-rank case of the reference benchmarks): straight-line batches of kFastBatch
+    // chunks, peer loads double-buffered one batch ahead across slab boundaries.
+    if constexpr (!F32) {
+        constexpr int kFastPeers = 7;
+        constexpr int kFastBatch = BM >= 256 ? 2 : 1;   // chunks per batch (the small tile keeps two workgroups per CU)
+        constexpr int kFastBatches = EP_ITERS / kFastBatch;
+        static_assert(kFastBatches % 2 == 0, "the two peer buffers alternate with a static parity");
+        if (EVEN && g.n_peers == kFastPeers && wave_m0 >= band_lo && wave_m0 + WTM <= band_hi) {
+            u32x4 pv[2][kFastBatch][kFastPeers];
+            const uint16_t* peer_base = g.peers + ((int64_t)(wave_m0 - band_lo + lane_r) * g.N + n);
+            const int64_t chunk_step = (int64_t)(64 / CPR) * g.N;   // elements between consecutive chunks of a lane
+            auto issue = [&](auto buf_c, int chunk_abs) __attribute__((always_inline)) {
+                constexpr int buf = decltype(buf_c)::value;
+#pragma unroll
+                for (int c = 0; c < kFastBatch; ++c)
+#pragma unroll
+                    for (int q = 0; q < kFastPeers; ++q)
+                        pv[buf][c][q] =
+                            ld_stream((const u32x4*)(peer_base + q * g.peers_stride + (chunk_abs + c) * chunk_step));
+            };
+            issue(std::integral_constant<int, 0>{}, 0);
+#pragma nounroll
+            for (int i = 0; i < TM; ++i) {
+                copy_slab(i);
+                const int chunk0 = i * EP_ITERS;   // chunks are numbered through all slabs of the wave
+#pragma unroll
+                for (int b = 0; b < kFastBatches; ++b) {
+                    // unconditional (the very last batch re-fetches itself, unused): a prefetch under
+                    // a branch would make the wait below assume the shorter queue and stall on stores
+                    const int next_chunk = min(chunk0 + (b + 1) * kFastBatch, TM * EP_ITERS - kFastBatch);
+                    if (b & 1) issue(std::integral_constant<int, 0>{}, next_chunk);
+                    else issue(std::integral_constant<int, 1>{}, next_chunk);
+                    float f[kFastBatch][8];
+#pragma unroll
+                    for (int c = 0; c < kFastBatch; ++c) read_chunk(b * kFastBatch + c, f[c]);
+#pragma unroll
+                    for (int c = 0; c < kFastBatch; ++c) {
+#pragma unroll
+                        for (int q = 0; q < kFastPeers; ++q) add8(pv[b & 1][c][q], f[c]);
+#pragma unroll
+                        for (int e = 0; e < 8; ++e) f[c][e] += bias_f[e];
+                    }
+#pragma unroll
+                    for (int c = 0; c < kFastBatch; ++c) {
+                        const int m = wave_m0 + (chunk0 + b * kFastBatch + c) * (64 / CPR) + lane_r;
+                        store_out((int64_t)(m - band_lo) * g.N + n, f[c]);
+                    }
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+            }
+            return;
+        }
+    }
+
+    // ---- every other case, one slab at a time ------------------------------------------------
+    // One batch of kChunkBatch chunks of the current slab.  NP == 0: every row of the slab lies
+    // in the band and there are no peers; NP == -2: no row of the slab lies in the band (both
+    // straight-line code without loads); NP == -1: generic per-lane handling (band edge inside
+    // the slab, ragged tile, any peer count).
+    auto slab_batch = [&](auto np_c, int slab_m0, int b0) __attribute__((always_inline)) {
+        constexpr int NP = decltype(np_c)::value;
+        int64_t off[kChunkBatch];
+        bool in_band[kChunkBatch], valid[kChunkBatch];
+#pragma unroll
+        for (int c = 0; c < kChunkBatch; ++c) {
+            const int m = slab_m0 + (b0 + c) * (64 / CPR) + lane_r;
+            valid[c] = EVEN || (m < g.M && n < g.N);
+            in_band[c] = NP == 0 ? true : NP == -2 ? false : (valid[c] && m >= band_lo && m < band_hi);
+            off[c] = in_band[c] ? (int64_t)(m - band_lo) * g.N + n : (int64_t)m * g.N + n;
+        }
+        if constexpr (!F32 && NP != -1) {
+            // nothing to add but perhaps the bias: the bf16 chunks go out as they are
+            if (NP == -2 || !has_bias) {
+                if (NP == 0 || g.c_full != nullptr) {
+                    uint16_t* dst = NP == 0 ? (uint16_t*)g.out : g.c_full;
+#pragma unroll
+                    for (int c = 0; c < kChunkBatch; ++c) st_stream((u32x4*)(dst + off[c]), read_raw(b0 + c));
+                }
+                return;
+            }
+        }
+        float f[kChunkBatch][8];
+#pragma unroll
+        for (int c = 0; c < kChunkBatch; ++c) read_chunk(b0 + c, f[c]);
+        if constexpr (NP == -1) {
+            // Peers in groups of kPeerGroup, all loads of a group issued before its first add;
+            // the groups are unrolled, each under one uniform test.  No load is predicated:
+            // a chunk outside the band reads a valid in-band address instead, a peer index
+            // past the last repeats the last peer, and such values are masked to +0.0 (loads
+            // under branches would make every later load wait for the whole queue).
+            const int64_t safe_off = min(n, g.N - 8);
+#pragma unroll
+            for (int q0 = 0; q0 < KR_MAX_WORLD - 1; q0 += kPeerGroup) {
+                if (q0 < g.n_peers) {
+                    u32x4 pv[kChunkBatch][kPeerGroup];
+#pragma unroll
+                    for (int c = 0; c < kChunkBatch; ++c)
+#pragma unroll
+                        for (int q = 0; q < kPeerGroup; ++q) {
+                            const int qq = min(q0 + q, g.n_peers - 1);
+                            pv[c][q] = ld_stream(
+                                (const u32x4*)(g.peers + qq * g.peers_stride + (in_band[c] ? off[c] : safe_off)));
+                        }
+#pragma unroll
+                    for (int c = 0; c < kChunkBatch; ++c)
+#pragma unroll
+                        for (int q = 0; q < kPeerGroup; ++q) {
+                            const uint32_t keep = (in_band[c] && q0 + q < g.n_peers) ? 0xffffffffu : 0u;
+                            add8(u32x4{pv[c][q].x & keep, pv[c][q].y & keep, pv[c][q].z & keep, pv[c][q].w & keep}, f[c]);
+                        }
+                }
+            }
+        }
+#pragma unroll
+        for (int c = 0; c < kChunkBatch; ++c) {
+            if (in_band[c]) {
+#pragma unroll
+                for (int e = 0; e < 8; ++e) f[c][e] += bias_f[e];
+                store_out(off[c], f[c]);
+            } else if (valid[c] && g.c_full != nullptr) {
+                st_stream((u32x4*)(g.c_full + off[c]), pack8(f[c]));
+            }
+        }
+    };
+
+#pragma nounroll
+    for (int i = 0; i < TM; ++i) {
+        copy_slab(i);
         const int slab_m0 = wave_m0 + i * 32;
         const bool all_in = EVEN && slab_m0 >= band_lo && slab_m0 + 32 <= band_hi;
         const bool all_out = EVEN && (slab_m0 + 32 <= band_lo || slab_m0 >= band_hi);
@@ -202,8 +305,6 @@ __device__ __forceinline__ void gemm_epilogue(const GemmArgs& g, const f32x16 (&
         for (int b0 = 0; b0 < EP_ITERS; b0 += kChunkBatch) {
             if (all_out) {
                 slab_batch(std::integral_constant<int, -2>{}, slab_m0, b0);
-            } else if (all_in && g.n_peers == 7) {
-                slab_batch(std::integral_constant<int, 7>{}, slab_m0, b0);
             } else if (all_in && g.n_peers == 0) {
                 slab_batch(std::integral_constant<int, 0>{}, slab_m0, b0);
             } else {
@@ -212,6 +313,13 @@ __device__ __forceinline__ void gemm_epilogue(const GemmArgs& g, const f32x16 (&
             __builtin_amdgcn_sched_barrier(0);
         }
     }
+}
+
+template <int BM, int WTM, int WTN, int TM, int TN, bool EVEN, int EP_WAVE>
+__device__ __forceinline__ void gemm_epilogue(const GemmArgs& g, const f32x16 (&acc)[TM][TN], unsigned char* smem,
+                                              int m0, int n0, int wm, int wn, int lane, int wave) {
+    if (g.out_is_fp32) gemm_epilogue_impl<true, BM, WTM, WTN, TM, TN, EVEN, EP_WAVE>(g, acc, smem, m0, n0, wm, wn, lane, wave);
+    else gemm_epilogue_impl<false, BM, WTM, WTN, TM, TN, EVEN, EP_WAVE>(g, acc, smem, m0, n0, wm, wn, lane, wave);
 }
 
 }  // namespace kr

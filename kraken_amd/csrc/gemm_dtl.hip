@@ -35,8 +35,7 @@ constexpr int B_ST = BN * BKD * 2;            // 16 KiB
 constexpr uint32_t B_BASE = NSTAGE * A_ST;    // 64 KiB
 constexpr int LDS_BYTES = NSTAGE * (A_ST + B_ST);
 constexpr int LOADS_PER_TILE = 8;             // LDS-DMA loads per wave per k-step (4 A + 4 B)
-constexpr int EP_LD = WTN + 4;
-constexpr int EP_WAVE = 32 * EP_LD * 4;
+constexpr int EP_WAVE = 32 * (WTN + 4) * 4;     // epilogue patch of a wave: 32 rows x WTN fp32, padded
 static_assert(EP_WAVE * WM * WN <= LDS_BYTES, "epilogue patch must fit in the operand ring");
 
 typedef __attribute__((address_space(3))) void* lds_void;
@@ -47,6 +46,7 @@ typedef __attribute__((address_space(3))) s16x4* lds_tr;
 // s_waitcnt vmcnt(n) only (expcnt and lgkmcnt left at "no wait")
 constexpr int vmcnt_imm(int n) { return (n & 15) | (7 << 4) | (15 << 8) | ((n >> 4) << 14); }
 constexpr int kLgkm0 = 0xc07f;   // s_waitcnt lgkmcnt(0) only
+
 
 template <bool B_NT>
 __global__ __launch_bounds__(WM* WN * 64) void gemm_dtl_kernel(const GemmArgs g) {
@@ -193,7 +193,7 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_dtl_kernel(const GemmArgs g)
 #pragma unroll
         for (int s = 0; s < NM; ++s) {
             const int i = s / TN, j = s % TN;
-            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[0][i], bfr[0][j], acc[i][j], 0, 0, 0);
+            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bfr[0][j], af[0][i], acc[i][j], 0, 0, 0);
             // fragments of sub-step 1, this stage: A blocks next to MFMAs 0..3, B blocks 4..7 / 4..11
             if (s < TM) read_a(1, s, 1, st_cur);
             else if (s < TM + TN) read_b(1, s - TM, 1, st_cur);
@@ -202,16 +202,19 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_dtl_kernel(const GemmArgs g)
                 __builtin_amdgcn_s_waitcnt(vmcnt_imm(LOADS_PER_TILE));
                 __builtin_amdgcn_s_barrier();
             }
-            if (s >= 4 && s < 4 + LOADS_PER_TILE) issue_load(t + 3, s - 4);
+            // one load every third MFMA (continued in sub-step 1): four waves issuing a load per
+            // MFMA ask twice what the CU's address unit takes, and the waves stall at issue
+            if (s >= 4 && (s - 4) % 3 == 0 && (s - 4) / 3 < LOADS_PER_TILE / 2) issue_load(t + 3, (s - 4) / 3);
             KR_SCHED_FENCE();
         }
 #pragma unroll
         for (int s = 0; s < NM; ++s) {
             const int i = s / TN, j = s % TN;
-            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[1][i], bfr[1][j], acc[i][j], 0, 0, 0);
+            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bfr[1][j], af[1][i], acc[i][j], 0, 0, 0);
             // first fragments of k-step t+1 (its stage is complete since the barrier above)
             if (s < TM) read_a(0, s, 0, st_nxt);
             else if (s < TM + TN) read_b(0, s - TM, 0, st_nxt);
+            if (s % 3 == 0 && s / 3 < LOADS_PER_TILE / 2) issue_load(t + 3, LOADS_PER_TILE / 2 + s / 3);
             KR_SCHED_FENCE();
         }
     }
@@ -220,7 +223,7 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_dtl_kernel(const GemmArgs g)
     __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));
     __syncthreads();
 
-    gemm_epilogue<BM, WTM, WTN, TM, TN, true, EP_LD, EP_WAVE>(g, acc, smem, m0, n0, wm, wn, lane, wave);
+    gemm_epilogue<BM, WTM, WTN, TM, TN, true, EP_WAVE>(g, acc, smem, m0, n0, wm, wn, lane, wave);
 }
 
 }  // namespace

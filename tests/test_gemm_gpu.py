@@ -13,12 +13,11 @@ BF16 = torch.bfloat16
 TOL = dict(rtol=2e-2, atol=2e-2)
 
 
-@pytest.fixture(params=["128", "256-staged", "256-lds-dma"])
+@pytest.fixture(params=["128", "256"])
 def tile(request, monkeypatch):
-    """Force each GEMM kernel in turn: 128x128 tiles; 256x256 tiles with the register-staged main
-    loop; 256x256 tiles with direct global->LDS loads (shapes a kernel cannot take fall back)."""
-    monkeypatch.setenv("KRAKEN_AMD_GEMM_TILE", request.param[:3])
-    monkeypatch.setenv("KRAKEN_AMD_GEMM_PATH", "staged" if request.param.endswith("staged") else "dtl")
+    """Force each GEMM kernel in turn: the register-staged kernel with 128x128 tiles; the
+    LDS-DMA kernel with 256x256 tiles (shapes it cannot take fall back to the other)."""
+    monkeypatch.setenv("KRAKEN_AMD_GEMM_TILE", request.param)
     return request.param
 
 
@@ -144,7 +143,6 @@ def _sampled_rows_check(got, rows, a, b, extra, tol=TOL):
 def test_baseline_config4_full_size(dev, monkeypatch):
     """A [8192,3584] @ B [3584,8192]; band of 1024 rows + 7 partials.  Oracle on sampled rows."""
     monkeypatch.delenv("KRAKEN_AMD_GEMM_TILE", raising=False)
-    monkeypatch.delenv("KRAKEN_AMD_GEMM_PATH", raising=False)
     M, N, K, W, rank = 8192, 8192, 3584, 8, 3
     a = orc.randn_bf16((M, K), 42)
     b = orc.randn_bf16((K, N), 43, 0.02)
@@ -165,7 +163,6 @@ def test_baseline_config4_full_size(dev, monkeypatch):
 
 def test_baseline_config5_full_size(dev, monkeypatch):
     monkeypatch.delenv("KRAKEN_AMD_GEMM_TILE", raising=False)
-    monkeypatch.delenv("KRAKEN_AMD_GEMM_PATH", raising=False)
     # fused all-reduce: A [4096,1024] @ B [1024,8192] + 7 partials + bias
     M, N, K, P = 4096, 8192, 1024, 7
     a = orc.randn_bf16((M, K), 42)
