@@ -417,6 +417,10 @@ extern "C" int kr_gemm_reduce_bf16(const void* A, int64_t lda_m, int64_t lda_k, 
         if (t[0] == '2') big = true;
     }
     const bool dtl = big && gemm_dtl_supported(g);
+    // KRAKEN_AMD_GEMM_PEERS=epilogue keeps the peers' partial sums out of the matrix cores
+    // (they are then added in the epilogue, where a non-finite value stays in its element)
+    g.peers_on_mfma = 1;
+    if (const char* t = getenv("KRAKEN_AMD_GEMM_PEERS")) g.peers_on_mfma = t[0] == 'e' ? 0 : t[0] == 'f' ? 2 : t[0] == 'l' ? 3 : 1;
     const int bm = dtl ? 256 : 128, bn = bm;
     g.tiles_m = (int)((M + bm - 1) / bm);
     g.tiles_n = (int)((N + bn - 1) / bn);

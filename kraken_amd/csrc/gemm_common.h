@@ -23,6 +23,7 @@ struct GemmArgs {
     int out_is_fp32;
     int pivot_tiles;   // rotation of the M-tile order
     int tiles_m, tiles_n;
+    int peers_on_mfma;   // 256x256 kernel: add whole-band tiles' peers through the matrix cores
 };
 
 // LDS-DMA kernel for shapes the 256x256 tile divides (gemm_dtl.hip)
@@ -104,11 +105,19 @@ __device__ __forceinline__ void gemm_epilogue_impl(const GemmArgs& g, const f32x
     if (has_bias) add8(*(const u32x4*)(g.bias + (EVEN ? n : min(n, g.N - 8))), bias_f);
 
     // Round-to-nearest-even pack of two fp32 to bf16, pinned where it is written: the
-    // accumulators do not change inside the slab loop, so an ordinary conversion would be
-    // hoisted out of it for all slabs at once, at the price of 128 more live registers.
+    // accumulators do not change inside the slab loop, so an ordinary conversion -- or, for
+    // accumulators held in AGPRs, even just the copy to a VALU-readable register -- would be
+    // hoisted out of it for all slabs at once, at the price of 128 or more live registers.
     auto pack_here = [](float lo, float hi) __attribute__((always_inline)) {
         uint32_t r;
-        asm volatile("v_cvt_pk_bf16_f32 %0, %1, %2" : "=v"(r) : "v"(lo), "v"(hi));
+        if constexpr (BM >= 256) {   // 256 accumulators: they live in AGPRs
+            uint32_t t;
+            asm volatile("v_accvgpr_read_b32 %0, %2\n\tv_accvgpr_read_b32 %1, %3\n\tv_cvt_pk_bf16_f32 %0, %0, %1"
+                         : "=&v"(r), "=&v"(t)
+                         : "a"(lo), "a"(hi));
+        } else {
+            asm volatile("v_cvt_pk_bf16_f32 %0, %1, %2" : "=v"(r) : "v"(lo), "v"(hi));
+        }
         return r;
     };
     // copy of slab i's accumulators to the patch.  Accumulator registers can only be indexed

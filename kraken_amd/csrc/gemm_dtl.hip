@@ -48,10 +48,10 @@ constexpr int vmcnt_imm(int n) { return (n & 15) | (7 << 4) | (15 << 8) | ((n >>
 constexpr int kLgkm0 = 0xc07f;   // s_waitcnt lgkmcnt(0) only
 
 
-template <bool B_NT>
-__global__ __launch_bounds__(WM* WN * 64) void gemm_dtl_kernel(const GemmArgs g) {
-    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];   // starts at LDS address 0
-
+// One workgroup tile.  PEERS_FIRST picks the order of the two accumulation phases (peers'
+// partial sums, k loop) for tiles whose peers are added on the matrix cores.
+template <bool B_NT, bool PEERS_FIRST>
+__device__ __forceinline__ void gemm_dtl_tile(const GemmArgs& g, unsigned char* smem) {
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -166,6 +166,99 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_dtl_kernel(const GemmArgs g)
             for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
 
 #define KR_SCHED_FENCE() __builtin_amdgcn_sched_barrier(0)
+    // ---- partial sums of the other ranks, added on the matrix cores ---------------------------
+    // For a tile that lies in the reduce band as a whole, the peers' partial sums P_q[m][n] are
+    // accumulated into the same registers as the product, as  acc[n][m] += sum_k X_h[n][k] *
+    // P_q[m][16h + k]  with X_h[n][k] = (n == 16h + k): the second MFMA operand wants, per lane,
+    // 8 consecutive n of one row m -- 16 contiguous bytes of the peer's row-major buffer.  Each
+    // wave streams its 128 x 128 part of every peer through a private quarter of the operand
+    // ring (four stages of 32 rows x 256 B, filled by LDS-DMA four items ahead, 16-byte pieces
+    // XOR-swizzled with the row so the fragment reads are conflict-free).  1.0 * bf16 products
+    // and the fp32 accumulation are exact, so this is the fp32 sum  product + P_0 + ... + P_{W-2}
+    // rounded once -- but 0 * Inf = NaN: a non-finite partial sum spoils the 16 columns of its
+    // row that share its MFMA, not just its own element.
+    // The phase is bound by HBM, the k loop by the matrix cores: workgroups alternate the order
+    // of the two, so at any time about half the CUs stream peers while the other half multiply.
+    const int band_lo = g.band_row0;
+    const bool mfma_peers = g.peers_on_mfma && g.n_peers > 0 && m0 >= band_lo && m0 + BM <= band_lo + g.band_rows;
+    auto peer_phase = [&]() __attribute__((always_inline)) {
+        constexpr int kItemLoads = 8;          // 1 KiB LDS-DMA loads per item (32 rows x 256 B)
+        constexpr int kItemBytes = kItemLoads * 1024;
+        constexpr int kAhead = 4;              // items in flight = stages per wave
+        static_assert(TM == 4 && kAhead * kItemBytes * WM * WN <= LDS_BYTES, "peer stages must fit in the ring");
+        typedef short s16x8 __attribute__((ext_vector_type(8)));
+        bf16x8 xid[2];
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            s16x8 x;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) x[e] = ((lane & 31) == 16 * h + 8 * (lane >> 5) + e) ? (short)0x3f80 : (short)0;
+            xid[h] = __builtin_bit_cast(bf16x8, x);
+        }
+        const uint32_t region = (uint32_t)wave * (kAhead * kItemBytes);
+        // load r of an item fills rows 4r .. 4r+3: lane l -> row 4r + l/16, piece slot l%16 holds
+        // piece slot ^ (row & 15); r = 4a + b puts 16a rows into the scalar offset
+        uint32_t pvoff[4];
+#pragma unroll
+        for (int b = 0; b < 4; ++b) {
+            const int row = 4 * b + (lane >> 4);
+            pvoff[b] = (uint32_t)(((int64_t)row * g.N + (((lane & 15) ^ row) << 3)) * 2);
+        }
+        // fragment (j, h): lane l -> row l%32, piece 4j + 2h + l/32
+        uint32_t pa[2 * TN];
+#pragma unroll
+        for (int jh = 0; jh < 2 * TN; ++jh) {
+            const int row = lane & 31;
+            pa[jh] = region + (uint32_t)(row * 256 + (((2 * jh + (lane >> 5)) ^ (row & 15)) << 4));
+        }
+        const int n_items = g.n_peers * TM;    // item = (peer q, slab i), q-major
+        const uint16_t* wave_base = g.peers + ((int64_t)(m0 + wm * WTM - band_lo) * g.N + n0 + wn * WTN);
+        auto issue_item = [&](int it, int stage) __attribute__((always_inline)) {
+            const int itc = min(it, n_items - 1);   // past the end: re-request the last item, unused
+            const i32x4 rs = make_rsrc(wave_base + (int64_t)(itc >> 2) * g.peers_stride + (int64_t)(itc & 3) * 32 * g.N);
+#pragma unroll
+            for (int r = 0; r < kItemLoads; ++r)
+                lds_dma_b128(rs, region + stage * kItemBytes + r * 1024, pvoff[r & 3], (int)((int64_t)(r >> 2) * 16 * g.N * 2));
+        };
+#pragma unroll
+        for (int it = 0; it < kAhead; ++it) issue_item(it, it);
+#pragma nounroll
+        for (int q = 0; q < g.n_peers; ++q) {
+#pragma unroll
+            for (int i = 0; i < TM; ++i) {
+                // item (q, i) has landed when at most the three younger items are outstanding; the
+                // stages are private to the wave, so no barrier
+                __builtin_amdgcn_s_waitcnt(vmcnt_imm((kAhead - 1) * kItemLoads));
+                KR_SCHED_FENCE();
+                bf16x8 y[2 * TN];
+#pragma unroll
+                for (int jh = 0; jh < 2 * TN; ++jh) y[jh] = *(lds_frag)(size_t)(pa[jh] + i * kItemBytes);
+                KR_SCHED_FENCE();   // all eight reads in flight before the first MFMA waits for one
+#pragma unroll
+                for (int jh = 0; jh < 2 * TN; ++jh)
+                    acc[i][jh >> 1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(xid[jh & 1], y[jh], acc[i][jh >> 1], 0, 0, 0);
+                // every fragment read has returned before the stage is handed back to the DMA
+                __builtin_amdgcn_s_waitcnt(kLgkm0);
+                KR_SCHED_FENCE();
+                issue_item(q * TM + i + kAhead, i);
+                KR_SCHED_FENCE();
+            }
+        }
+        __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));
+        __syncthreads();   // the ring is handed on (k loop or epilogue patches of other waves)
+    };
+    // An empty statement that names every accumulator as an AGPR operand, placed between the
+    // phases: with the live ranges cut here the register allocator keeps the accumulators
+    // where the MFMAs left them instead of moving them to VGPRs and memory for the next phase.
+    auto pin_accumulators = [&]() __attribute__((always_inline)) {
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+            for (int j = 0; j < TN; ++j) asm volatile("" : "+a"(acc[i][j]));
+    };
+    if (PEERS_FIRST && mfma_peers) peer_phase();
+    pin_accumulators();
+
     // ---- prologue: request k-steps 0, 1, 2; wait for step 0 ------------------------------------
 #pragma unroll
     for (int t = 0; t < 3; ++t)
@@ -218,12 +311,27 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_dtl_kernel(const GemmArgs g)
             KR_SCHED_FENCE();
         }
     }
-#undef KR_SCHED_FENCE
     // drain the tail's surplus loads before the LDS is reused
     __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));
     __syncthreads();
 
-    gemm_epilogue<BM, WTM, WTN, TM, TN, true, EP_WAVE>(g, acc, smem, m0, n0, wm, wn, lane, wave);
+    pin_accumulators();
+    if (!PEERS_FIRST && mfma_peers) peer_phase();
+    pin_accumulators();
+    GemmArgs ge = g;
+    if (mfma_peers) ge.n_peers = 0;   // already in the accumulators
+    gemm_epilogue<BM, WTM, WTN, TM, TN, true, EP_WAVE>(ge, acc, smem, m0, n0, wm, wn, lane, wave);
+}
+#undef KR_SCHED_FENCE
+
+// The two phase orders are two complete copies of the tile code under one uniform branch: each
+// copy is straight-line (phase, phase, epilogue), which keeps the 256 accumulators in their
+// registers; one copy with a run-time order has the register allocator move them through memory.
+template <bool B_NT>
+__global__ __launch_bounds__(WM* WN * 64) void gemm_dtl_kernel(const GemmArgs g) {
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];   // starts at LDS address 0
+    if (g.peers_on_mfma && g.n_peers > 0 && (g.peers_on_mfma == 1 ? ((blockIdx.x >> 3) & 1) : g.peers_on_mfma == 2)) gemm_dtl_tile<B_NT, true>(g, smem);
+    else gemm_dtl_tile<B_NT, false>(g, smem);
 }
 
 }  // namespace

@@ -13,11 +13,14 @@ BF16 = torch.bfloat16
 TOL = dict(rtol=2e-2, atol=2e-2)
 
 
-@pytest.fixture(params=["128", "256"])
+@pytest.fixture(params=["128", "256", "256-epilogue"])
 def tile(request, monkeypatch):
     """Force each GEMM kernel in turn: the register-staged kernel with 128x128 tiles; the
-    LDS-DMA kernel with 256x256 tiles (shapes it cannot take fall back to the other)."""
-    monkeypatch.setenv("KRAKEN_AMD_GEMM_TILE", request.param)
+    LDS-DMA kernel with 256x256 tiles (shapes it cannot take fall back to the other), with the
+    peers' partial sums of whole-band tiles added on the matrix cores (default) or in the
+    epilogue."""
+    monkeypatch.setenv("KRAKEN_AMD_GEMM_TILE", request.param[:3])
+    monkeypatch.setenv("KRAKEN_AMD_GEMM_PEERS", "epilogue" if request.param.endswith("epilogue") else "mfma")
     return request.param
 
 
@@ -143,6 +146,7 @@ def _sampled_rows_check(got, rows, a, b, extra, tol=TOL):
 def test_baseline_config4_full_size(dev, monkeypatch):
     """A [8192,3584] @ B [3584,8192]; band of 1024 rows + 7 partials.  Oracle on sampled rows."""
     monkeypatch.delenv("KRAKEN_AMD_GEMM_TILE", raising=False)
+    monkeypatch.delenv("KRAKEN_AMD_GEMM_PEERS", raising=False)
     M, N, K, W, rank = 8192, 8192, 3584, 8, 3
     a = orc.randn_bf16((M, K), 42)
     b = orc.randn_bf16((K, N), 43, 0.02)
@@ -163,6 +167,7 @@ def test_baseline_config4_full_size(dev, monkeypatch):
 
 def test_baseline_config5_full_size(dev, monkeypatch):
     monkeypatch.delenv("KRAKEN_AMD_GEMM_TILE", raising=False)
+    monkeypatch.delenv("KRAKEN_AMD_GEMM_PEERS", raising=False)
     # fused all-reduce: A [4096,1024] @ B [1024,8192] + 7 partials + bias
     M, N, K, P = 4096, 8192, 1024, 7
     a = orc.randn_bf16((M, K), 42)
