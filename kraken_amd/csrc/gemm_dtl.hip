@@ -66,16 +66,16 @@ __device__ __forceinline__ void gemm_dtl_tile(const GemmArgs& g, unsigned char* 
     // A / transposed B: chunk = 16 rows; lane l -> row l/4, slot l%4 holds chunk slot ^ ((row>>2)&3).
     // Only the wave-uniform part (chunk row, k) changes between loads: it goes to the scalar
     // offset; the per-lane byte offset is computed once.
-    const uint32_t a_voff =
+    const uint32_t a_voff_lane =
         (uint32_t)(((int64_t)(lane >> 2) * g.lda + (((lane & 3) ^ ((lane >> 4) & 3)) << 3)) * 2);
-    uint32_t b_voff;
+    uint32_t b_voff_lane;
     if (B_NT) {
-        b_voff = (uint32_t)(((int64_t)(lane >> 2) * g.ldb + (((lane & 3) ^ ((lane >> 4) & 3)) << 3)) * 2);
+        b_voff_lane = (uint32_t)(((int64_t)(lane >> 2) * g.ldb + (((lane & 3) ^ ((lane >> 4) & 3)) << 3)) * 2);
     } else {
         // row-major B: chunk = 2 k-rows of 512 B; lane l -> k-row l/32, piece slot l%32 holds piece
         // slot ^ 4*(k & 3); k & 3 = 2*(chunk & 1) + l/32 and chunk & 1 == wave & 1
         const int kq = ((wave & 1) << 1) | (lane >> 5);
-        b_voff = (uint32_t)(((int64_t)(lane >> 5) * g.ldb + (((lane & 31) ^ (kq << 2)) << 3)) * 2);
+        b_voff_lane = (uint32_t)(((int64_t)(lane >> 5) * g.ldb + (((lane & 31) ^ (kq << 2)) << 3)) * 2);
     }
     // Buffer resource descriptor: 48-bit base, stride 0 (raw), 2^31-1 bytes, 32-bit data format.
     typedef int i32x4 __attribute__((ext_vector_type(4)));
@@ -99,8 +99,13 @@ __device__ __forceinline__ void gemm_dtl_tile(const GemmArgs& g, unsigned char* 
     const int kt_total = g.K / BKD;
     // one LDS-DMA load of k-step t (clamped: the tail re-requests the last tile into a free stage)
     auto issue_load = [&](int t, int q) {
+        // past the end nothing new is needed, but the per-step load count must not change (the
+        // vmcnt arithmetic relies on it): every lane then re-reads the first 16 bytes of the
+        // last tile's chunk into the free stage -- one cache line instead of a kilobyte
+        const bool live = t < kt_total;
         const int tt = min(t, kt_total - 1);
         const int k0 = tt * BKD;
+        const uint32_t a_voff = live ? a_voff_lane : 0u, b_voff = live ? b_voff_lane : 0u;
         const uint32_t stage = (uint32_t)(t & (NSTAGE - 1));
         const int ch = wave + 4 * (q & 3);
         if (q < 4) {
@@ -214,11 +219,15 @@ __device__ __forceinline__ void gemm_dtl_tile(const GemmArgs& g, unsigned char* 
         const int n_items = g.n_peers * TM;    // item = (peer q, slab i), q-major
         const uint16_t* wave_base = g.peers + ((int64_t)(m0 + wm * WTM - band_lo) * g.N + n0 + wn * WTN);
         auto issue_item = [&](int it, int stage) __attribute__((always_inline)) {
-            const int itc = min(it, n_items - 1);   // past the end: re-request the last item, unused
+            // past the end: all lanes re-read 16 bytes of the last item (the load count per item
+            // is fixed for the vmcnt arithmetic; the data is never used)
+            const bool live = it < n_items;
+            const int itc = min(it, n_items - 1);
             const i32x4 rs = make_rsrc(wave_base + (int64_t)(itc >> 2) * g.peers_stride + (int64_t)(itc & 3) * 32 * g.N);
 #pragma unroll
             for (int r = 0; r < kItemLoads; ++r)
-                lds_dma_b128(rs, region + stage * kItemBytes + r * 1024, pvoff[r & 3], (int)((int64_t)(r >> 2) * 16 * g.N * 2));
+                lds_dma_b128(rs, region + stage * kItemBytes + r * 1024, live ? pvoff[r & 3] : 0u,
+                             live ? (int)((int64_t)(r >> 2) * 16 * g.N * 2) : 0);
         };
 #pragma unroll
         for (int it = 0; it < kAhead; ++it) issue_item(it, it);
