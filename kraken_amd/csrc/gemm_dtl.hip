@@ -52,6 +52,11 @@ constexpr int kLgkm0 = 0xc07f;   // s_waitcnt lgkmcnt(0) only
 // partial sums, k loop) for tiles whose peers are added on the matrix cores.
 template <bool B_NT, bool PEERS_FIRST>
 __device__ __forceinline__ void gemm_dtl_tile(const GemmArgs& g, unsigned char* smem) {
+    // Nothing is outstanding at kernel entry; saying so keeps the compiler's own wait-count
+    // bookkeeping from carrying the pending loads and stores of the other copy of this code
+    // (which never runs in the same workgroup) into this one, where it cannot see the LDS-DMA
+    // loads retire them and would re-wait for them in every k-step.
+    __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -88,7 +93,8 @@ __device__ __forceinline__ void gemm_dtl_tile(const GemmArgs& g, unsigned char* 
     // s_waitcnt vmcnt / s_barrier pairs below (told about it, it waits for vmcnt(0) in front of
     // every transposing LDS read, which serialises the whole pipeline).
     auto lds_dma_b128 = [](i32x4 rsrc, uint32_t lds_addr, uint32_t voff, int soff) {
-        asm volatile("s_mov_b32 m0, %0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
+        // (one wait state between the scalar write of M0 and the LDS-DMA instruction that reads it)
+        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
                      :
                      : "s"(lds_addr), "v"(voff), "s"(rsrc), "s"(soff)
                      : "memory", "m0");
