@@ -90,7 +90,7 @@ def _rand_sets(shape, nsets, dev, std=1.0, seed=1234):
 
 
 class OneShotReduce(Workload):
-    """BASELINE config 2: stack [8,4096,4096] -> [4096,4096]."""
+    """benchmark config 2: stack [8,4096,4096] -> [4096,4096]."""
     name = "one_shot_reduce_w8_4096x4096"
     R, D = 4096, 4096
     nsets = 4   # 4 x 256 MiB of input: no step finds its input in the 256 MB last-level cache
@@ -103,7 +103,7 @@ class OneShotReduce(Workload):
         from oracle import oracle as orc
 
         self.dev = dev
-        self.host = orc.make_stack(W, (self.R, self.D), seed0=42)       # the BASELINE inputs, set 0
+        self.host = orc.make_stack(W, (self.R, self.D), seed0=42)       # the benchmark inputs, set 0
         self.sets = [self.host.to(dev)] + _rand_sets((W, self.R, self.D), self.nsets - 1, dev)
         self.out = None
 
@@ -132,7 +132,7 @@ class OneShotReduce(Workload):
 
 
 class TwoShotShare(OneShotReduce):
-    """BASELINE config 2, two-shot variant: this rank's 1/8 row chunk [512,4096]."""
+    """benchmark config 2, two-shot variant: this rank's 1/8 row chunk [512,4096]."""
     name = "two_shot_share_w8_512x4096"
     nsets = 4
     use_graph = True      # ~6 us kernel: replay the timed steps from a HIP graph
@@ -161,7 +161,7 @@ class TwoShotShare(OneShotReduce):
 
 
 class ReduceBiasRmsNorm(Workload):
-    """BASELINE configs 1 and 3 (and a large-row variant that fills the GPU)."""
+    """benchmark configs 1 and 3 (and a large-row variant that fills the GPU)."""
 
     def __init__(self, rows, D, nsets, tag):
         self.rows, self.D, self.nsets = rows, D, nsets
@@ -206,7 +206,7 @@ class ReduceBiasRmsNorm(Workload):
 
 
 class GemmReduceScatter(Workload):
-    """BASELINE config 4: A [8192,3584] @ B [3584,8192]; own 1024-row band + 7 partials."""
+    """benchmark config 4: A [8192,3584] @ B [3584,8192]; own 1024-row band + 7 partials."""
     name = "gemm_reduce_scatter_8192x8192x3584_w8"
     bound = "mfma"
     M, N, K = 8192, 8192, 3584
@@ -257,7 +257,7 @@ class GemmReduceScatter(Workload):
 
 
 class GemmAllReduce(Workload):
-    """BASELINE config 5 (fused): A [4096,1024] @ B [1024,8192] + 7 partials + bias; HBM-bound."""
+    """benchmark config 5 (fused): A [4096,1024] @ B [1024,8192] + 7 partials + bias; HBM-bound."""
     name = "gemm_all_reduce_4096x8192x1024_w8"
     bound = "hbm"
     M, N, K = 4096, 8192, 1024
@@ -308,7 +308,7 @@ class GemmAllReduce(Workload):
 
 
 class AllGatherMatmul(Workload):
-    """BASELINE config 5 (all-gather): A stack [8,1024,8192] @ B [8192,3584], B.T contiguous."""
+    """benchmark config 5 (all-gather): A stack [8,1024,8192] @ B [8192,3584], B.T contiguous."""
     name = "all_gather_matmul_8192x3584x8192_w8"
     bound = "mfma"
     m, K, N = 1024, 8192, 3584

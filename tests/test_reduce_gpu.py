@@ -145,7 +145,7 @@ def test_rotated_band_reduce(dev):
 
 
 def test_full_size_config2(dev):
-    """BASELINE config 2: stack [8,4096,4096] -> [4096,4096], and the two-shot 1/8 row chunk.
+    """benchmark config 2: stack [8,4096,4096] -> [4096,4096], and the two-shot 1/8 row chunk.
     Checked exactly against the oracle on sampled row bands, and by linearity on the whole."""
     W, R, D = 8, 4096, 4096
     g = torch.Generator(device="cpu"); g.manual_seed(42)
