@@ -168,13 +168,42 @@ __device__ __forceinline__ void gemm_dtl_tile(const GemmArgs& g, unsigned char* 
         }
     };
 
+    // The accumulators start at the bias instead of zero when the whole tile lies in the reduce
+    // band and nothing is left for the epilogue to add in bf16 (no peers, or peers added on the
+    // matrix cores): product, partial sums and bias are then summed in fp32 and rounded once,
+    // and the epilogue just converts and stores.  Lane holds row m; register v of block j is
+    // column 32j + 8(v/4) + 4(lane/32) + v%4, so a lane needs 16 groups of 4 consecutive bias
+    // values, the same for all four row blocks.
+    const int band_lo = g.band_row0;
+    const bool tile_in_band = m0 >= band_lo && m0 + BM <= band_lo + g.band_rows;
+    const bool mfma_peers = g.peers_on_mfma && g.n_peers > 0 && tile_in_band;
+    const bool bias_in_acc = g.bias != nullptr && tile_in_band && (g.n_peers == 0 || mfma_peers);
     f32x16 acc[TM][TN];
-#pragma unroll
-    for (int i = 0; i < TM; ++i)
+    {
+        f32x16 init[TN];
 #pragma unroll
         for (int j = 0; j < TN; ++j)
 #pragma unroll
-            for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
+            for (int v = 0; v < 16; ++v) init[j][v] = 0.0f;
+        if (bias_in_acc) {
+            typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+            const uint16_t* bp = g.bias + n0 + wn * WTN + 4 * (lane >> 5);
+#pragma unroll
+            for (int j = 0; j < TN; ++j)
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    const u32x2 b4 = *(const u32x2*)(bp + j * 32 + 8 * q);
+                    init[j][4 * q + 0] = bf16_lo(b4.x);
+                    init[j][4 * q + 1] = bf16_hi(b4.x);
+                    init[j][4 * q + 2] = bf16_lo(b4.y);
+                    init[j][4 * q + 3] = bf16_hi(b4.y);
+                }
+        }
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+            for (int j = 0; j < TN; ++j) acc[i][j] = init[j];
+    }
 
 #define KR_SCHED_FENCE() __builtin_amdgcn_sched_barrier(0)
     // ---- partial sums of the other ranks, added on the matrix cores ---------------------------
@@ -190,8 +219,6 @@ __device__ __forceinline__ void gemm_dtl_tile(const GemmArgs& g, unsigned char* 
     // row that share its MFMA, not just its own element.
     // The phase is bound by HBM, the k loop by the matrix cores: workgroups alternate the order
     // of the two, so at any time about half the CUs stream peers while the other half multiply.
-    const int band_lo = g.band_row0;
-    const bool mfma_peers = g.peers_on_mfma && g.n_peers > 0 && m0 >= band_lo && m0 + BM <= band_lo + g.band_rows;
     auto peer_phase = [&]() __attribute__((always_inline)) {
         constexpr int kItemLoads = 8;          // 1 KiB LDS-DMA loads per item (32 rows x 256 B)
         constexpr int kItemBytes = kItemLoads * 1024;
@@ -335,6 +362,7 @@ __device__ __forceinline__ void gemm_dtl_tile(const GemmArgs& g, unsigned char* 
     pin_accumulators();
     GemmArgs ge = g;
     if (mfma_peers) ge.n_peers = 0;   // already in the accumulators
+    if (bias_in_acc) ge.bias = nullptr;
     gemm_epilogue<BM, WTM, WTN, TM, TN, true, EP_WAVE>(ge, acc, smem, m0, n0, wm, wn, lane, wave);
 }
 #undef KR_SCHED_FENCE
