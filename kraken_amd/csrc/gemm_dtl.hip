@@ -99,6 +99,13 @@ __device__ __forceinline__ void gemm_dtl_tile(const GemmArgs& g, unsigned char* 
                      : "s"(lds_addr), "v"(voff), "s"(rsrc), "s"(soff)
                      : "memory", "m0");
     };
+    // same with the non-temporal hint, for data that is read exactly once (the peers' sums)
+    auto lds_dma_b128_stream = [](i32x4 rsrc, uint32_t lds_addr, uint32_t voff, int soff) {
+        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen nt lds"
+                     :
+                     : "s"(lds_addr), "v"(voff), "s"(rsrc), "s"(soff)
+                     : "memory", "m0");
+    };
     const i32x4 a_rsrc = make_rsrc(g.A + (int64_t)m0 * g.lda);
     const i32x4 bt_rsrc = make_rsrc(g.B + (int64_t)n0 * g.ldb);
 
@@ -259,7 +266,7 @@ __device__ __forceinline__ void gemm_dtl_tile(const GemmArgs& g, unsigned char* 
             const i32x4 rs = make_rsrc(wave_base + (int64_t)(itc >> 2) * g.peers_stride + (int64_t)(itc & 3) * 32 * g.N);
 #pragma unroll
             for (int r = 0; r < kItemLoads; ++r)
-                lds_dma_b128(rs, region + stage * kItemBytes + r * 1024, live ? pvoff[r & 3] : 0u,
+                lds_dma_b128_stream(rs, region + stage * kItemBytes + r * 1024, live ? pvoff[r & 3] : 0u,
                              live ? (int)((int64_t)(r >> 2) * 16 * g.N * 2) : 0);
         };
 #pragma unroll
