@@ -66,11 +66,12 @@ __device__ __forceinline__ void tile_schedule(const GemmArgs& g, int& tile_m_out
 // contiguous store into a row-major LDS patch.  `smem` is the workgroup's LDS (free for reuse:
 // every wave has passed a barrier after its last read of the operand stages).
 //
-// F32 = false (bf16 result): the product is rounded to bf16 on its way into the patch, exactly
-// as the reference rounds a rank's partial product before it is summed
-// (kraken/fused/gemm_one_shot_all_reduce_fused.py:120-135); partial sums of the peers and the
-// bias are then added in fp32 in the order own, peer 0, 1, ..., bias.
-// F32 = true (fp32 result, used by the split-fp32 emulation): the patch holds fp32.
+// F32 = false (bf16 result): the product is rounded to bf16 on its way into the patch, as the
+// reference's reduce-scatter rounds a rank's partial product before the partials are summed
+// (kraken/fused/gemm_reduce_scatter_fused.py:72, summed in fp32 at :118-145); partial sums of
+// the peers and the bias are then added in fp32 in the order own, peer 0, 1, ..., bias.
+// F32 = true (fp32 result: the reference's fused all-reduce keeps fp32 from the accumulator to
+// the output, kraken/fused/gemm_one_shot_all_reduce_fused.py:65-99): the patch holds fp32.
 template <bool F32, int BM, int WTM, int WTN, int TM, int TN, bool EVEN, int EP_WAVE>
 __device__ __forceinline__ void gemm_epilogue_impl(const GemmArgs& g, const f32x16 (&acc)[TM][TN], unsigned char* smem,
                                                    int m0, int n0, int wm, int wn, int lane, int wave) {

@@ -14,12 +14,18 @@
 //     then touch all 64 banks once.
 //   row-major B: [32 k][512 B] (256 n), the 16-byte pieces of a k-row XOR-swizzled with
 //     4*(k & 3): the 32 lanes of two neighbouring 16-lane blocks (4 k-rows x 32 columns) then
-//     cover 16 different pieces = all 64 banks.  Fragments are read with ds_read_b64_tr_b16: 16 lanes read a 4(k) x 16(n)
-//     block, four n each, and the hardware hands lane i the four k of column i -- two such
-//     reads give the eight k per lane the MFMA wants, with no transpose in registers.
+//     cover 16 different pieces = all 64 banks.  Fragments are read with ds_read_b64_tr_b16:
+//     16 lanes read a 4(k) x 16(n) block, four n each, and the hardware hands lane i the four
+//     k of column i -- two such reads give the eight k per lane the MFMA wants, with no
+//     transpose in registers.
 // A lane's fragment addresses differ between the 32x32 blocks, the two 16-wide k sub-steps
 // and the stages only by compile-time constants, so they are immediate offsets on two (A),
 // two (B transposed) or four (B row-major) address registers.
+//
+// The B fragment is the first MFMA operand and the A fragment the second, so the accumulators
+// hold C transposed: a lane owns one row m and four consecutive columns n per register quad,
+// which is what the fused epilogue (gemm_common.h) stores and what lets the partial sums of the
+// other ranks be added by the matrix cores themselves (peer_phase below).
 #include "gemm_common.h"
 
 namespace kr {
@@ -46,7 +52,6 @@ typedef __attribute__((address_space(3))) s16x4* lds_tr;
 // s_waitcnt vmcnt(n) only (expcnt and lgkmcnt left at "no wait")
 constexpr int vmcnt_imm(int n) { return (n & 15) | (7 << 4) | (15 << 8) | ((n >> 4) << 14); }
 constexpr int kLgkm0 = 0xc07f;   // s_waitcnt lgkmcnt(0) only
-
 
 // One workgroup tile.  PEERS_FIRST picks the order of the two accumulation phases (peers'
 // partial sums, k loop) for tiles whose peers are added on the matrix cores.
@@ -327,7 +332,7 @@ __device__ __forceinline__ void gemm_dtl_tile(const GemmArgs& g, unsigned char* 
     // first fragments of k-step t+1 are read into buffer 0.  After the first MFMAs of the step
     // the wave waits until its own loads of step t+1 have landed (those of step t+2 may still be
     // in flight) and meets the other waves: from then on step t+1 is complete in LDS and the
-    // stage of step t-1 is free, so the loads of step t+3 go out, one next to each MFMA.
+    // stage of step t-1 is free, so the loads of step t+3 go out, one every third MFMA.
     constexpr int NM = TM * TN;
     for (int t = 0; t < kt_total; ++t) {
         const uint32_t st_cur = (uint32_t)(t & (NSTAGE - 1)) * A_ST;
