@@ -192,3 +192,22 @@ def test_baseline_config5_full_size(dev, monkeypatch):
     _sampled_rows_check(c, rows, stack.reshape(W * m, K2), bT.T, None)
     ref = stack.to(dev).reshape(W * m, K2).float() @ bT.to(dev).T.float()
     torch.testing.assert_close(c.float(), ref.to(BF16).float(), **TOL)
+
+
+def test_all_gather_matmul_reference_test_shape(dev, monkeypatch):
+    """test/test_allgather_matmul.py:51-66: M=4096, N=6656, K=16384, bf16, B.T contiguous, here with W=8 shards of
+    512 rows; the gathered A must be the exact stack, C within the gate of the sampled-row oracle
+    and of the device's fp32 GEMM on the whole matrix."""
+    monkeypatch.delenv("KRAKEN_AMD_GEMM_TILE", raising=False)
+    monkeypatch.delenv("KRAKEN_AMD_GEMM_PEERS", raising=False)
+    W, M, N, K = 8, 4096, 6656, 16384
+    stack = orc.make_stack(W, (M // W, K), seed0=42)
+    bT = orc.randn_bf16((N, K), 43, 0.02)
+    sd = stack.to(dev)
+    for rank in (0, 5):
+        ag, c = fused.all_gather_matmul(sd, bT.to(dev).T, rank=rank)
+        assert torch.equal(ag.cpu(), stack.reshape(M, K))
+        rows = torch.tensor([0, 511, 512, 5 * 512 + 3, 4095])
+        _sampled_rows_check(c, rows, stack.reshape(M, K), bT.T, None)
+        ref = sd.reshape(M, K).float() @ bT.to(dev).T.float()
+        torch.testing.assert_close(c.float(), ref.to(BF16).float(), **TOL)
