@@ -35,10 +35,11 @@ namespace {
 constexpr int BM = 256, BN = 256, WM = 2, WN = 2;
 constexpr int WTM = BM / WM, WTN = BN / WN, TM = WTM / 32, TN = WTN / 32;
 constexpr int BKD = 32;                       // k extent of one stage
-constexpr int NSTAGE = 4;
+constexpr int NSTAGE = 4;                     // LDS ring depth: tiles are requested NSTAGE-1 k-steps ahead
+                                              // (a fifth stage, all 160 KiB, measured no faster)
 constexpr int A_ST = BM * BKD * 2;            // 16 KiB
 constexpr int B_ST = BN * BKD * 2;            // 16 KiB
-constexpr uint32_t B_BASE = NSTAGE * A_ST;    // 64 KiB
+constexpr uint32_t B_BASE = NSTAGE * A_ST;
 constexpr int LDS_BYTES = NSTAGE * (A_ST + B_ST);
 constexpr int LOADS_PER_TILE = 8;             // LDS-DMA loads per wave per k-step (4 A + 4 B)
 constexpr int EP_WAVE = 32 * (WTN + 4) * 4;     // epilogue patch of a wave: 32 rows x WTN fp32, padded
@@ -116,7 +117,7 @@ __device__ __forceinline__ void gemm_dtl_tile(const GemmArgs& g, unsigned char* 
 
     const int kt_total = g.K / BKD;
     // one LDS-DMA load of k-step t (clamped: the tail re-requests the last tile into a free stage)
-    auto issue_load = [&](int t, int q) {
+    auto issue_load = [&](int t, uint32_t stage, int q) {
         // past the end nothing new is needed, but the per-step load count must not change (the
         // vmcnt arithmetic relies on it): every lane then re-reads the first 16 bytes of the
         // last tile's chunk into the free stage -- one cache line instead of a kilobyte
@@ -124,7 +125,6 @@ __device__ __forceinline__ void gemm_dtl_tile(const GemmArgs& g, unsigned char* 
         const int tt = min(t, kt_total - 1);
         const int k0 = tt * BKD;
         const uint32_t a_voff = live ? a_voff_lane : 0u, b_voff = live ? b_voff_lane : 0u;
-        const uint32_t stage = (uint32_t)(t & (NSTAGE - 1));
         const int ch = wave + 4 * (q & 3);
         if (q < 4) {
             lds_dma_b128(a_rsrc, stage * A_ST + ch * 1024, a_voff, (int)(((int64_t)16 * ch * g.lda + k0) * 2));
@@ -313,12 +313,12 @@ __device__ __forceinline__ void gemm_dtl_tile(const GemmArgs& g, unsigned char* 
     if (PEERS_FIRST && mfma_peers) peer_phase();
     pin_accumulators();
 
-    // ---- prologue: request k-steps 0, 1, 2; wait for step 0 ------------------------------------
+    // ---- prologue: request k-steps 0 .. NSTAGE-2; wait for step 0 -----------------------------
 #pragma unroll
-    for (int t = 0; t < 3; ++t)
+    for (int t = 0; t < NSTAGE - 1; ++t)
 #pragma unroll
-        for (int q = 0; q < LOADS_PER_TILE; ++q) issue_load(t, q);
-    __builtin_amdgcn_s_waitcnt(vmcnt_imm(2 * LOADS_PER_TILE));
+        for (int q = 0; q < LOADS_PER_TILE; ++q) issue_load(t, (uint32_t)t, q);
+    __builtin_amdgcn_s_waitcnt(vmcnt_imm((NSTAGE - 2) * LOADS_PER_TILE));
     __builtin_amdgcn_s_barrier();
     KR_SCHED_FENCE();
 #pragma unroll
@@ -330,13 +330,16 @@ __device__ __forceinline__ void gemm_dtl_tile(const GemmArgs& g, unsigned char* 
     // k-step t: 2 sub-steps of 16 MFMAs.  Sub-step 0 computes on fragment buffer 0 while the
     // fragments of sub-step 1 are read into buffer 1; sub-step 1 computes on buffer 1 while the
     // first fragments of k-step t+1 are read into buffer 0.  After the first MFMAs of the step
-    // the wave waits until its own loads of step t+1 have landed (those of step t+2 may still be
-    // in flight) and meets the other waves: from then on step t+1 is complete in LDS and the
-    // stage of step t-1 is free, so the loads of step t+3 go out, one every third MFMA.
+    // the wave waits until its own loads of step t+1 have landed (those of the later steps may
+    // still be in flight) and meets the other waves: from then on step t+1 is complete in LDS
+    // and the stage of step t-1 is free, so the loads of step t+NSTAGE-1 go out into it, one
+    // every third MFMA.
     constexpr int NM = TM * TN;
+    uint32_t stage_cur = 0;   // t % NSTAGE
     for (int t = 0; t < kt_total; ++t) {
-        const uint32_t st_cur = (uint32_t)(t & (NSTAGE - 1)) * A_ST;
-        const uint32_t st_nxt = (uint32_t)((t + 1) & (NSTAGE - 1)) * A_ST;
+        const uint32_t stage_nxt = stage_cur + 1 == NSTAGE ? 0 : stage_cur + 1;
+        const uint32_t stage_ld = stage_cur == 0 ? NSTAGE - 1 : stage_cur - 1;   // (t + NSTAGE - 1) % NSTAGE
+        const uint32_t st_cur = stage_cur * A_ST, st_nxt = stage_nxt * A_ST;
 #pragma unroll
         for (int s = 0; s < NM; ++s) {
             const int i = s / TN, j = s % TN;
@@ -346,12 +349,12 @@ __device__ __forceinline__ void gemm_dtl_tile(const GemmArgs& g, unsigned char* 
             else if (s < TM + TN) read_b(1, s - TM, 1, st_cur);
             if (s == 3) {
                 KR_SCHED_FENCE();
-                __builtin_amdgcn_s_waitcnt(vmcnt_imm(LOADS_PER_TILE));
+                __builtin_amdgcn_s_waitcnt(vmcnt_imm((NSTAGE - 3) * LOADS_PER_TILE));
                 __builtin_amdgcn_s_barrier();
             }
             // one load every third MFMA (continued in sub-step 1): four waves issuing a load per
             // MFMA ask twice what the CU's address unit takes, and the waves stall at issue
-            if (s >= 4 && (s - 4) % 3 == 0 && (s - 4) / 3 < LOADS_PER_TILE / 2) issue_load(t + 3, (s - 4) / 3);
+            if (s >= 4 && (s - 4) % 3 == 0 && (s - 4) / 3 < LOADS_PER_TILE / 2) issue_load(t + NSTAGE - 1, stage_ld, (s - 4) / 3);
             KR_SCHED_FENCE();
         }
 #pragma unroll
@@ -361,9 +364,10 @@ __device__ __forceinline__ void gemm_dtl_tile(const GemmArgs& g, unsigned char* 
             // first fragments of k-step t+1 (its stage is complete since the barrier above)
             if (s < TM) read_a(0, s, 0, st_nxt);
             else if (s < TM + TN) read_b(0, s - TM, 0, st_nxt);
-            if (s % 3 == 0 && s / 3 < LOADS_PER_TILE / 2) issue_load(t + 3, LOADS_PER_TILE / 2 + s / 3);
+            if (s % 3 == 0 && s / 3 < LOADS_PER_TILE / 2) issue_load(t + NSTAGE - 1, stage_ld, LOADS_PER_TILE / 2 + s / 3);
             KR_SCHED_FENCE();
         }
+        stage_cur = stage_nxt;
     }
     // drain the tail's surplus loads before the LDS is reused
     __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));
@@ -392,7 +396,7 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_dtl_kernel(const GemmArgs g)
 }  // namespace
 
 bool gemm_dtl_supported(const GemmArgs& g) {
-    return g.M % BM == 0 && g.N % BN == 0 && g.K % BKD == 0 && g.K >= 3 * BKD &&
+    return g.M % BM == 0 && g.N % BN == 0 && g.K % BKD == 0 && g.K >= (NSTAGE - 1) * BKD &&
            (int64_t)BM * g.lda * 2 < 0x7fffffffLL && (int64_t)(BN > 64 ? BN : 64) * g.ldb * 2 < 0x7fffffffLL;
 }
 
