@@ -335,8 +335,9 @@ __device__ __forceinline__ void gemm_dtl_tile(const GemmArgs& g, unsigned char* 
     // and the stage of step t-1 is free, so the loads of step t+NSTAGE-1 go out into it, one
     // every third MFMA.
     constexpr int NM = TM * TN;
-    uint32_t stage_cur = 0;   // t % NSTAGE
-    for (int t = 0; t < kt_total; ++t) {
+    // one k-step; `stage_c` is t % NSTAGE, as a compile-time constant in the unrolled loop
+    auto k_step = [&](int t, auto stage_c) __attribute__((always_inline)) {
+        const uint32_t stage_cur = stage_c;
         const uint32_t stage_nxt = stage_cur + 1 == NSTAGE ? 0 : stage_cur + 1;
         const uint32_t stage_ld = stage_cur == 0 ? NSTAGE - 1 : stage_cur - 1;   // (t + NSTAGE - 1) % NSTAGE
         const uint32_t st_cur = stage_cur * A_ST, st_nxt = stage_nxt * A_ST;
@@ -367,7 +368,27 @@ __device__ __forceinline__ void gemm_dtl_tile(const GemmArgs& g, unsigned char* 
             if (s % 3 == 0 && s / 3 < LOADS_PER_TILE / 2) issue_load(t + NSTAGE - 1, stage_ld, LOADS_PER_TILE / 2 + s / 3);
             KR_SCHED_FENCE();
         }
-        stage_cur = stage_nxt;
+    };
+    // Main part: one trip = NSTAGE k-steps, so every LDS stage offset is a compile-time constant
+    // (immediate offsets on the fragment reads, no per-step address arithmetic) and the loop
+    // branch is taken once per NSTAGE steps.  The at most NSTAGE-1 remaining steps follow.
+    static_assert(NSTAGE == 4, "the unrolled trip below spells out four stages");
+    int t = 0;
+#pragma nounroll
+    for (; t + NSTAGE <= kt_total; t += NSTAGE) {
+        k_step(t, std::integral_constant<uint32_t, 0>{});
+        k_step(t + 1, std::integral_constant<uint32_t, 1>{});
+        k_step(t + 2, std::integral_constant<uint32_t, 2>{});
+        k_step(t + 3, std::integral_constant<uint32_t, 3>{});
+    }
+    pin_accumulators();
+    {
+        uint32_t stage_cur = 0;   // t is a multiple of NSTAGE here
+#pragma nounroll
+        for (; t < kt_total; ++t) {
+            k_step(t, stage_cur);
+            stage_cur = stage_cur + 1 == NSTAGE ? 0 : stage_cur + 1;
+        }
     }
     // drain the tail's surplus loads before the LDS is reused
     __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));
