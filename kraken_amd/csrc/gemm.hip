@@ -425,6 +425,15 @@ extern "C" int kr_gemm_reduce_bf16(const void* A, int64_t lda_m, int64_t lda_k, 
     g.tiles_m = (int)((M + bm - 1) / bm);
     g.tiles_n = (int)((N + bn - 1) / bn);
     if ((int64_t)g.tiles_m * g.tiles_n > 0x7fffffffLL) return KR_ERR_BAD_DIM;
+    // Column panels per scheduling group: the tiles an XCD runs at a time form a block that is
+    // group_n panels wide.  8 measured best for the compute-bound shapes; where most tiles also
+    // stream the peers' partial sums (HBM-bound), 16 lets neighbouring CUs read longer runs of
+    // the same rows at about the same time.
+    g.group_n = (n_peers > 0 && band_rows * 2 >= M) ? 16 : 8;
+    if (const char* t = getenv("KRAKEN_AMD_GEMM_GROUP")) {
+        const int v = atoi(t);
+        if (v >= 1 && v <= 64) g.group_n = v;
+    }
     int64_t pt = tile_pivot / bm;
     g.pivot_tiles = (int)(((pt % g.tiles_m) + g.tiles_m) % g.tiles_m);
     const bool even = (M % bm == 0 && N % bn == 0 && K % BK == 0);

@@ -23,6 +23,7 @@ struct GemmArgs {
     int out_is_fp32;
     int pivot_tiles;   // rotation of the M-tile order
     int tiles_m, tiles_n;
+    int group_n;         // column panels per scheduling group (tile_schedule)
     int peers_on_mfma;   // 256x256 kernel: add whole-band tiles' peers through the matrix cores
 };
 
@@ -30,7 +31,6 @@ struct GemmArgs {
 bool gemm_dtl_supported(const GemmArgs& g);
 hipError_t launch_gemm_dtl(const GemmArgs& g, bool b_nt, hipStream_t st);
 
-constexpr int kGroupN = 4;        // column panels per scheduling group
 constexpr int kXcds = 8;
 
 // Map the workgroup id to its tile (tile_m, tile_n).
@@ -38,19 +38,19 @@ __device__ __forceinline__ void tile_schedule(const GemmArgs& g, int& tile_m_out
     // ---- tile schedule -------------------------------------------------------------------
     // Workgroups are dealt round-robin to the 8 XCDs (each with its own L2), so workgroup ids
     // are first re-numbered to give every XCD a contiguous range of tiles.  Tiles are then
-    // ordered in groups of kGroupN column panels, M fastest in steps of kGroupN columns: the
-    // ~32 tiles an XCD runs at a time form an 8 x 4 block that shares 8 A panels and 4 B
-    // panels through its L2, and every XCD works on all row bands -- the rows of the reduce
+    // ordered in groups of g.group_n column panels, M fastest in steps of g.group_n columns: the
+    // ~32 tiles an XCD runs at a time form a (32 / group_n) x group_n block that shares its A and
+    // B panels through the XCD's L2 (a dozen panels for 32 tiles), and every XCD works on all row bands -- the rows of the reduce
     // band (whose tiles also stream the peers' partial sums) are spread over all XCDs
     // instead of landing on one.  The M order is rotated by the pivot, so the band's (or the
     // local shard's) tiles are the first ones of every XCD.
     int pid = blockIdx.x;
     const int ntiles = g.tiles_m * g.tiles_n;
     if (ntiles % kXcds == 0) pid = (pid % kXcds) * (ntiles / kXcds) + pid / kXcds;
-    const int per_group = kGroupN * g.tiles_m;
+    const int per_group = g.group_n * g.tiles_m;
     const int group = pid / per_group;
-    const int first_n = group * kGroupN;
-    const int gsz = min(g.tiles_n - first_n, kGroupN);
+    const int first_n = group * g.group_n;
+    const int gsz = min(g.tiles_n - first_n, g.group_n);
     const int tile_n = first_n + (pid % per_group) % gsz;
     int tile_m = (pid % per_group) / gsz;
     tile_m += g.pivot_tiles;
