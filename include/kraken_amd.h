@@ -135,6 +135,14 @@ int kr_rmsnorm_bf16(const void* x, const void* w, float eps, int64_t rows, int64
  *        changes scheduling only, never the result.
  * Requirements: K % 8 == 0, N % 8 == 0, leading strides % 8 == 0, pointers
  * 16-byte aligned, 0 <= band_row0, band_row0 + band_rows <= M.
+ * Rounding: the sum is formed in fp32 and rounded once at the store; with a
+ * bf16 result, tiles whose peers are added in the epilogue round the product
+ * to bf16 before the sum, as gemm_reduce_scatter_fused.py:72 does.
+ * Non-finite input: for shapes the 256x256 kernel takes (M % 256 == N % 256
+ * == 0, K % 32 == 0) the peers of tiles lying wholly in the band are added
+ * on the matrix cores, where an Inf/NaN in a peer also turns the 15
+ * neighbouring columns of its row into NaN; KRAKEN_AMD_GEMM_PEERS=epilogue
+ * in the environment keeps such values in their own element.
  *
  * Replaces
  *   kraken/fused/gemm_one_shot_all_reduce_fused.py:56-99   (band = all rows)
