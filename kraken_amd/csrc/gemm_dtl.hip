@@ -227,7 +227,7 @@ __device__ __forceinline__ void gemm_dtl_tile(const GemmArgs& g, unsigned char* 
     // ring (four stages of 32 rows x 256 B, filled by LDS-DMA four items ahead, 16-byte pieces
     // XOR-swizzled with the row so the fragment reads are conflict-free).  1.0 * bf16 products
     // and the fp32 accumulation are exact, so this is the fp32 sum  product + P_0 + ... + P_{W-2}
-    // rounded once -- but 0 * Inf = NaN: a non-finite partial sum spoils the 16 columns of its
+    // rounded once -- but 0 * Inf = NaN: a non-finite partial sum spoils the 32-column block of its
     // row that share its MFMA, not just its own element.
     // The phase is bound by HBM, the k loop by the matrix cores: workgroups alternate the order
     // of the two, so at any time about half the CUs stream peers while the other half multiply.

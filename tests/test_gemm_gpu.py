@@ -211,3 +211,28 @@ def test_all_gather_matmul_reference_test_shape(dev, monkeypatch):
         _sampled_rows_check(c, rows, stack.reshape(M, K), bT.T, None)
         ref = sd.reshape(M, K).float() @ bT.to(dev).T.float()
         torch.testing.assert_close(c.float(), ref.to(BF16).float(), **TOL)
+
+
+@pytest.mark.parametrize("mode", ["mfma", "epilogue"])
+def test_non_finite_partial_sum_stays_local(dev, monkeypatch, mode):
+    """An Inf in one peer's partial sum: added in the epilogue it shows up in its own element
+    only; added on the matrix cores (identity MFMA, 0 * Inf = NaN) it may also spoil the columns
+    of its row that share its MFMA -- the aligned block of 32 -- and nothing else."""
+    monkeypatch.setenv("KRAKEN_AMD_GEMM_TILE", "256")
+    monkeypatch.setenv("KRAKEN_AMD_GEMM_PEERS", mode)
+    M, N, K, P = 512, 512, 256, 3
+    a, b, peers = mk(M, N, K, P)
+    r, c = 300, 77
+    peers[1, r, c] = float("inf")
+    out = fused.gemm_one_shot_all_reduce_fused(a.to(dev), b.to(dev), peers=peers.to(dev), out_dtype=BF16).cpu().float()
+    clean = peers.clone()
+    clean[1, r, c] = 0.0
+    want = orc.gemm_all_reduce(a, b, clean).to(BF16).float()
+    bad = ~torch.isfinite(out)
+    assert bad[r, c]
+    group = torch.zeros_like(bad)
+    group[r, c // 32 * 32:c // 32 * 32 + 32] = True
+    assert not (bad & ~group).any()
+    if mode == "epilogue":
+        assert bad.sum() == 1 and out[r, c] == float("inf")
+    torch.testing.assert_close(out[~group], want[~group], **TOL)
