@@ -236,3 +236,18 @@ def test_non_finite_partial_sum_stays_local(dev, monkeypatch, mode):
     if mode == "epilogue":
         assert bad.sum() == 1 and out[r, c] == float("inf")
     torch.testing.assert_close(out[~group], want[~group], **TOL)
+
+
+@pytest.mark.parametrize("P", [1, 2, 7, 8, 15])
+def test_gemm_all_reduce_world_sizes(dev, tile, P):
+    """Every world size the C ABI accepts (W = P + 1 up to 16), on a shape with whole-band
+    256-tiles (matrix-core or epilogue peer path) and on a ragged one (generic epilogue path)."""
+    for (M, N, K) in [(512, 256, 160), (200, 136, 72)]:
+        a, b, peers = mk(M, N, K, P, seed=P)
+        bias = orc.randn_bf16((N,), 9, 0.02)
+        want = orc.gemm_all_reduce(a, b, peers, bias)
+        out = fused.gemm_one_shot_all_reduce_fused(a.to(dev), b.to(dev), peers=peers.to(dev), bias=bias.to(dev))
+        torch.testing.assert_close(out.cpu(), want, rtol=1e-3, atol=1e-3)
+        outb = fused.gemm_one_shot_all_reduce_fused(a.to(dev), b.to(dev), peers=peers.to(dev), bias=bias.to(dev),
+                                                    out_dtype=BF16)
+        torch.testing.assert_close(outb.cpu(), want.to(BF16), **TOL)
