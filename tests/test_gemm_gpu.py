@@ -251,3 +251,38 @@ def test_gemm_all_reduce_world_sizes(dev, tile, P):
         outb = fused.gemm_one_shot_all_reduce_fused(a.to(dev), b.to(dev), peers=peers.to(dev), bias=bias.to(dev),
                                                     out_dtype=BF16)
         torch.testing.assert_close(outb.cpu(), want.to(BF16), **TOL)
+
+
+def test_gemm_paths_replay_from_a_graph(dev, monkeypatch):
+    """The GEMM entry point enqueues kernels only (no allocation, no memset, no host sync), so a
+    caller may capture it: three fused calls are captured once and replayed with eager work in
+    between; every replay must reproduce the eager result bit for bit."""
+    monkeypatch.delenv("KRAKEN_AMD_GEMM_TILE", raising=False)
+    monkeypatch.delenv("KRAKEN_AMD_GEMM_PEERS", raising=False)
+    M, N, K, W, rank = 1024, 512, 512, 4, 1
+    a, b, peers_full = mk(M, N, K, W - 1)
+    bias = orc.randn_bf16((N,), 3, 0.02)
+    ad, bd, bias_d = a.to(dev), b.to(dev), bias.to(dev)
+    bt = bd.T.contiguous().T               # all_gather_matmul wants b.T contiguous
+    pf = peers_full.to(dev)
+    pb = pf[:, :M // W].contiguous()
+    eager = (fused.gemm_one_shot_all_reduce_fused(ad, bd, peers=pf, bias=bias_d, out_dtype=BF16),
+             fused.gemm_reduce_scatter(ad, bd, peers=pb, rank=rank),
+             fused.all_gather_matmul(ad.view(W, M // W, K), bt, rank=rank)[1])
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(g, stream=side):
+            got = (fused.gemm_one_shot_all_reduce_fused(ad, bd, peers=pf, bias=bias_d, out_dtype=BF16),
+                   fused.gemm_reduce_scatter(ad, bd, peers=pb, rank=rank),
+                   fused.all_gather_matmul(ad.view(W, M // W, K), bt, rank=rank)[1])
+    for rep in range(3):
+        for t in got:
+            t.zero_()                      # eager work between the replays
+        torch.cuda.synchronize()
+        g.replay()
+        torch.cuda.synchronize()
+        for e, r in zip(eager, got):
+            assert torch.equal(e, r)
