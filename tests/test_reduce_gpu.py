@@ -164,3 +164,38 @@ def test_full_size_config2(dev):
     # swapping two slices leaves the result within one rounding
     sd2 = sd.clone(); sd2[[0, 7]] = sd[[7, 0]]
     torch.testing.assert_close(comm.one_shot_all_reduce(sd2).float(), out.float(), rtol=2 ** -7, atol=1e-5)
+
+
+def test_reduce_paths_replay_from_a_graph(dev):
+    """The reduce and row entry points enqueue kernels only: captured once, every replay (with
+    eager work in between) reproduces the eager result bit for bit."""
+    W, rows, D = 8, 48, 5120
+    stack = orc.make_stack(W, (rows, D)).to(dev)
+    bias, w = orc.make_bias_weight(D)
+    bias, w = bias.to(dev), w.to(dev)
+    out = torch.empty(rows, D, dtype=BF16, device=dev)
+    y = torch.empty(rows, D, dtype=BF16, device=dev)
+
+    def run():
+        s1 = comm.one_shot_all_reduce(stack)
+        s2 = comm.two_shot_all_reduce(stack, rank=2)
+        fused.one_shot_all_reduce_bias(stack, None, bias.expand(rows, D).contiguous(), out)
+        fused.one_shot_all_reduce_bias_rms_norm(stack, None, bias, w, y)
+        return s1, s2, out, y
+
+    eager = [t.clone() for t in run()]
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(g, stream=side):
+            got = run()
+    for rep in range(3):
+        for t in got:
+            t.zero_()
+        torch.cuda.synchronize()
+        g.replay()
+        torch.cuda.synchronize()
+        for e, r in zip(eager, got):
+            assert torch.equal(e, r)
