@@ -1,26 +1,29 @@
 // bf16 GEMM main loop with direct global->LDS loads ("LDS DMA") for shapes the 256x256 tile
-// divides:  M % 256 == 0, N % 256 == 0, K % 32 == 0.
+// divides:  M % 256 == 0, N % 256 == 0, K % 64 == 0.
 //
 // Workgroup tile 256 x 256, four wavefronts (2 x 2), each owning 128 x 128 of C as 4 x 4
-// v_mfma_f32_32x32x16_bf16 accumulators (256 AGPRs).  The k loop advances 32 at a time; the
-// operand tiles of four k-steps live in a ring of LDS stages (A: 4 x 16 KiB at 0, B: 4 x 16 KiB
-// at 64 KiB) that is filled by buffer_load ... lds: the data never passes through VGPRs, no
-// ds_write is issued, and a tile is requested three k-steps before it is used.
+// v_mfma_f32_32x32x16_bf16 accumulators (256 AGPRs).  The k loop advances 64 at a time through a
+// double buffer of LDS stages (A: 2 x 32 KiB at 0, B: 2 x 32 KiB at 64 KiB) that is filled by
+// buffer_load ... lds: the data never passes through VGPRs and no ds_write is issued.  With 64 k
+// per stage a row of A (or of transposed B) is 128 contiguous bytes, one L2 cache line per row
+// and load: a four-stage ring of 32-k stages, tried first, was more tolerant of load latency but
+// asked the L2 for every line twice (twice the L1-to-L2 requests of hipBLASLt's kernel in the
+// counters) and measured 3-7 % slower.
 //
 // LDS layouts (per stage)
-//   A and transposed-contiguous B: [256 rows][64 B] (32 k), the four 16-byte chunks of a row
-//     XOR-swizzled with (row >> 2) & 3.  One wave-wide LDS-DMA load fills 16 rows (1 KiB,
-//     lane l -> row l/4, chunk slot l%4); the 128-bit fragment reads of 16 consecutive rows
+//   A and transposed-contiguous B: [256 rows][128 B] (64 k), the eight 16-byte pieces of a row
+//     XOR-swizzled with (row >> 1) & 7.  One wave-wide LDS-DMA load fills 8 rows (1 KiB,
+//     lane l -> row l/8, piece slot l%8); the 128-bit fragment reads of 16 consecutive rows
 //     then touch all 64 banks once.
-//   row-major B: [32 k][512 B] (256 n), the 16-byte pieces of a k-row XOR-swizzled with
+//   row-major B: [64 k][512 B] (256 n), the 16-byte pieces of a k-row XOR-swizzled with
 //     4*(k & 3): the 32 lanes of two neighbouring 16-lane blocks (4 k-rows x 32 columns) then
 //     cover 16 different pieces = all 64 banks.  Fragments are read with ds_read_b64_tr_b16:
 //     16 lanes read a 4(k) x 16(n) block, four n each, and the hardware hands lane i the four
 //     k of column i -- two such reads give the eight k per lane the MFMA wants, with no
 //     transpose in registers.
-// A lane's fragment addresses differ between the 32x32 blocks, the two 16-wide k sub-steps
-// and the stages only by compile-time constants, so they are immediate offsets on two (A),
-// two (B transposed) or four (B row-major) address registers.
+// A lane's fragment addresses differ between the 32x32 blocks and the stages only by compile-time
+// constants (immediate offsets); the four 16-wide k sub-steps of a stage take one address
+// register each (A, B transposed) or an immediate (B row-major, one register per column block).
 //
 // The B fragment is the first MFMA operand and the A fragment the second, so the accumulators
 // hold C transposed: a lane owns one row m and four consecutive columns n per register quad,
@@ -34,14 +37,14 @@ namespace {
 
 constexpr int BM = 256, BN = 256, WM = 2, WN = 2;
 constexpr int WTM = BM / WM, WTN = BN / WN, TM = WTM / 32, TN = WTN / 32;
-constexpr int BKD = 32;                       // k extent of one stage
-constexpr int NSTAGE = 4;                     // LDS ring depth: tiles are requested NSTAGE-1 k-steps ahead
-                                              // (a fifth stage, all 160 KiB, measured no faster)
-constexpr int A_ST = BM * BKD * 2;            // 16 KiB
-constexpr int B_ST = BN * BKD * 2;            // 16 KiB
-constexpr uint32_t B_BASE = NSTAGE * A_ST;
+constexpr int BKD = 64;                       // k extent of one stage: 128-byte rows, one L2 line per row and load
+constexpr int NSTAGE = 2;                     // double buffer
+constexpr int A_ST = BM * BKD * 2;            // 32 KiB
+constexpr int B_ST = BN * BKD * 2;            // 32 KiB
+constexpr uint32_t B_BASE = NSTAGE * A_ST;    // 64 KiB
 constexpr int LDS_BYTES = NSTAGE * (A_ST + B_ST);
-constexpr int LOADS_PER_TILE = 8;             // LDS-DMA loads per wave per k-step (4 A + 4 B)
+constexpr int LOADS_A = A_ST / 1024 / (WM * WN);   // LDS-DMA loads (1 KiB each) per wave per k-step: 8 A ...
+constexpr int LOADS_PER_TILE = 2 * LOADS_A;        // ... + 8 B
 constexpr int EP_WAVE = 32 * (WTN + 4) * 4;     // epilogue patch of a wave: 32 rows x WTN fp32, padded
 static_assert(EP_WAVE * WM * WN <= LDS_BYTES, "epilogue patch must fit in the operand ring");
 
@@ -73,15 +76,16 @@ __device__ __forceinline__ void gemm_dtl_tile(const GemmArgs& g, unsigned char* 
     const int m0 = tile_m * BM, n0 = tile_n * BN;
 
     // ---- LDS-DMA addressing ----------------------------------------------------------------
-    // A wave loads the 1 KiB chunks  wave, wave+4, wave+8, wave+12  of a stage.
-    // A / transposed B: chunk = 16 rows; lane l -> row l/4, slot l%4 holds chunk slot ^ ((row>>2)&3).
-    // Only the wave-uniform part (chunk row, k) changes between loads: it goes to the scalar
-    // offset; the per-lane byte offset is computed once.
-    const uint32_t a_voff_lane =
-        (uint32_t)(((int64_t)(lane >> 2) * g.lda + (((lane & 3) ^ ((lane >> 4) & 3)) << 3)) * 2);
+    // A wave loads the 1 KiB chunks  wave, wave+4, ..., wave+28  of a stage.
+    // A / transposed B: chunk = 8 rows of 128 B; lane l -> row l/8, slot l%8 holds the 16-byte
+    // piece  slot ^ ((row >> 1) & 7)  of the row.  (row >> 1) & 7 = (4*chunk + l/16) & 7 and chunk
+    // has the parity of the wave, so the per-lane byte offset is computed once; the wave-uniform
+    // part (chunk row, k) goes to the scalar offset.
+    const int dma_sw = (4 * (wave & 1) + (lane >> 4)) & 7;
+    const uint32_t a_voff_lane = (uint32_t)(((int64_t)(lane >> 3) * g.lda + (((lane & 7) ^ dma_sw) << 3)) * 2);
     uint32_t b_voff_lane;
     if (B_NT) {
-        b_voff_lane = (uint32_t)(((int64_t)(lane >> 2) * g.ldb + (((lane & 3) ^ ((lane >> 4) & 3)) << 3)) * 2);
+        b_voff_lane = (uint32_t)(((int64_t)(lane >> 3) * g.ldb + (((lane & 7) ^ dma_sw) << 3)) * 2);
     } else {
         // row-major B: chunk = 2 k-rows of 512 B; lane l -> k-row l/32, piece slot l%32 holds piece
         // slot ^ 4*(k & 3); k & 3 = 2*(chunk & 1) + l/32 and chunk & 1 == wave & 1
@@ -125,12 +129,12 @@ __device__ __forceinline__ void gemm_dtl_tile(const GemmArgs& g, unsigned char* 
         const int tt = min(t, kt_total - 1);
         const int k0 = tt * BKD;
         const uint32_t a_voff = live ? a_voff_lane : 0u, b_voff = live ? b_voff_lane : 0u;
-        const int ch = wave + 4 * (q & 3);
-        if (q < 4) {
-            lds_dma_b128(a_rsrc, stage * A_ST + ch * 1024, a_voff, (int)(((int64_t)16 * ch * g.lda + k0) * 2));
+        const int ch = wave + 4 * (q % LOADS_A);
+        if (q < LOADS_A) {
+            lds_dma_b128(a_rsrc, stage * A_ST + ch * 1024, a_voff, (int)(((int64_t)8 * ch * g.lda + k0) * 2));
         } else if (B_NT) {
             lds_dma_b128(bt_rsrc, B_BASE + stage * B_ST + ch * 1024, b_voff,
-                         (int)(((int64_t)16 * ch * g.ldb + k0) * 2));
+                         (int)(((int64_t)8 * ch * g.ldb + k0) * 2));
         } else {
             // re-based on the first k-row of the step: the scalar offset stays small for any K
             lds_dma_b128(make_rsrc(g.B + (int64_t)k0 * g.ldb + n0), B_BASE + stage * B_ST + ch * 1024, b_voff,
@@ -139,17 +143,18 @@ __device__ __forceinline__ void gemm_dtl_tile(const GemmArgs& g, unsigned char* 
     };
 
     // ---- fragment addressing -----------------------------------------------------------------
-    // A (and transposed B): lane -> row (lane & 31) of the 32-row block, 8 k at chunk 2*ks + (lane>>5)
+    // A (and transposed B): lane -> row (lane & 31) of the 32-row block, 8 k at piece 2*ks + (lane>>5)
+    // of the row's eight, stored at piece ^ ((row >> 1) & 7) -- the same for all blocks (their rows
+    // differ by 32); the sub-step enters as an XOR of bits 5..6
     const int frow = lane & 31, fkc = lane >> 5;
-    const int fsw = (frow >> 2) & 3;            // same for all blocks: block rows differ by 32
-    // byte address at ks = 0; ks = 1 flips bit 5 (chunk ^ 2)
-    const uint32_t fa0 = (uint32_t)((wm * WTM + frow) * 64 + (((fsw & 2) | (fkc ^ (fsw & 1))) << 4));
-    const uint32_t fa1 = fa0 ^ 32u;
-    uint32_t fb[4];
+    const int fsw = (frow >> 1) & 7;
+    uint32_t fa[4], fb[4];
+#pragma unroll
+    for (int ks = 0; ks < 4; ++ks) fa[ks] = (uint32_t)((wm * WTM + frow) * 128 + (((2 * ks + fkc) ^ fsw) << 4));
     if (B_NT) {
-        fb[0] = B_BASE + (uint32_t)((wn * WTN + frow) * 64 + (((fsw & 2) | (fkc ^ (fsw & 1))) << 4));
-        fb[1] = fb[0] ^ 32u;
-        fb[2] = fb[3] = 0;
+#pragma unroll
+        for (int ks = 0; ks < 4; ++ks)
+            fb[ks] = B_BASE + (uint32_t)((wn * WTN + frow) * 128 + (((2 * ks + fkc) ^ fsw) << 4));
     } else {
         // transposing read: 16-lane block b = lane/16, i = lane%16 reads k-row 8*(b>>1) + i/4,
         // columns 16*(b&1) + 4*(i%4) .. +3 of the 32-column block j
@@ -165,11 +170,11 @@ __device__ __forceinline__ void gemm_dtl_tile(const GemmArgs& g, unsigned char* 
 
     bf16x8 af[2][TM], bfr[2][TN];
     auto read_a = [&](int buf, int i, int ks, uint32_t stage_off) {
-        af[buf][i] = *(lds_frag)(size_t)((ks ? fa1 : fa0) + stage_off + i * 2048);
+        af[buf][i] = *(lds_frag)(size_t)(fa[ks] + stage_off + i * 4096);
     };
     auto read_b = [&](int buf, int j, int ks, uint32_t stage_off) {
         if (B_NT) {
-            bfr[buf][j] = *(lds_frag)(size_t)((ks ? fb[1] : fb[0]) + stage_off + j * 2048);
+            bfr[buf][j] = *(lds_frag)(size_t)(fb[ks] + stage_off + j * 4096);
         } else {
             const uint32_t a = fb[j] + stage_off + ks * 8192;
             const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_tr)(size_t)a);
@@ -313,12 +318,19 @@ __device__ __forceinline__ void gemm_dtl_tile(const GemmArgs& g, unsigned char* 
     if (PEERS_FIRST && mfma_peers) peer_phase();
     pin_accumulators();
 
-    // ---- prologue: request k-steps 0 .. NSTAGE-2; wait for step 0 -----------------------------
+    // ---- prologue: request k-step 0 and the first loads of step 1; wait for step 0 ------------
+    // How the LOADS_PER_TILE loads of a k-step are spread: kEarly go out right behind the barrier
+    // that frees their stage (rest of sub-step 3 of step t-2), the others during sub-steps 0 and
+    // 1 of step t-1 -- every second MFMA.  One per MFMA from four waves is twice what the CU's
+    // address unit takes (the waves then stall at issue); spreading them evenly over the whole
+    // step leaves the last ones too little time before the barrier that needs them.
+    constexpr int kEarly = 6;
+    static_assert(NSTAGE == 2 && LOADS_PER_TILE == 16, "load schedule below: 6 + 8 + 2 loads");
 #pragma unroll
-    for (int t = 0; t < NSTAGE - 1; ++t)
+    for (int q = 0; q < LOADS_PER_TILE; ++q) issue_load(0, 0, q);
 #pragma unroll
-        for (int q = 0; q < LOADS_PER_TILE; ++q) issue_load(t, (uint32_t)t, q);
-    __builtin_amdgcn_s_waitcnt(vmcnt_imm((NSTAGE - 2) * LOADS_PER_TILE));
+    for (int q = 0; q < kEarly; ++q) issue_load(1, 1, q);
+    __builtin_amdgcn_s_waitcnt(vmcnt_imm(kEarly));
     __builtin_amdgcn_s_barrier();
     KR_SCHED_FENCE();
 #pragma unroll
@@ -327,69 +339,58 @@ __device__ __forceinline__ void gemm_dtl_tile(const GemmArgs& g, unsigned char* 
     for (int j = 0; j < TN; ++j) read_b(0, j, 0, 0);
 
     // ---- main loop ---------------------------------------------------------------------------
-    // k-step t: 2 sub-steps of 16 MFMAs.  Sub-step 0 computes on fragment buffer 0 while the
-    // fragments of sub-step 1 are read into buffer 1; sub-step 1 computes on buffer 1 while the
-    // first fragments of k-step t+1 are read into buffer 0.  After the first MFMAs of the step
-    // the wave waits until its own loads of step t+1 have landed (those of the later steps may
-    // still be in flight) and meets the other waves: from then on step t+1 is complete in LDS
-    // and the stage of step t-1 is free, so the loads of step t+NSTAGE-1 go out into it, one
-    // every third MFMA.
+    // k-step t (64 k): 4 sub-steps of 16 MFMAs on alternating fragment buffers; sub-step ks
+    // computes on buffer ks&1 while the fragments of the next sub-step are read into the other.
+    // The fragments of sub-step 3 are read during sub-step 2, so when a wave has issued the first
+    // MFMAs of sub-step 3 every LDS read of the stage has returned: there it waits for its own
+    // loads of step t+1 and meets the other waves.  From then on stage t+1 is complete (its first
+    // fragments are read next) and stage t is free for the loads of step t+2.
     constexpr int NM = TM * TN;
-    // one k-step; `stage_c` is t % NSTAGE, as a compile-time constant in the unrolled loop
     auto k_step = [&](int t, auto stage_c) __attribute__((always_inline)) {
         const uint32_t stage_cur = stage_c;
-        const uint32_t stage_nxt = stage_cur + 1 == NSTAGE ? 0 : stage_cur + 1;
-        const uint32_t stage_ld = stage_cur == 0 ? NSTAGE - 1 : stage_cur - 1;   // (t + NSTAGE - 1) % NSTAGE
+        const uint32_t stage_nxt = stage_cur ^ 1u;
         const uint32_t st_cur = stage_cur * A_ST, st_nxt = stage_nxt * A_ST;
 #pragma unroll
-        for (int s = 0; s < NM; ++s) {
-            const int i = s / TN, j = s % TN;
-            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bfr[0][j], af[0][i], acc[i][j], 0, 0, 0);
-            // fragments of sub-step 1, this stage: A blocks next to MFMAs 0..3, B blocks 4..7 / 4..11
-            if (s < TM) read_a(1, s, 1, st_cur);
-            else if (s < TM + TN) read_b(1, s - TM, 1, st_cur);
-            if (s == 3) {
-                KR_SCHED_FENCE();
-                __builtin_amdgcn_s_waitcnt(vmcnt_imm((NSTAGE - 3) * LOADS_PER_TILE));
-                __builtin_amdgcn_s_barrier();
-            }
-            // one load every third MFMA (continued in sub-step 1): four waves issuing a load per
-            // MFMA ask twice what the CU's address unit takes, and the waves stall at issue
-            if (s >= 4 && (s - 4) % 3 == 0 && (s - 4) / 3 < LOADS_PER_TILE / 2) issue_load(t + NSTAGE - 1, stage_ld, (s - 4) / 3);
-            KR_SCHED_FENCE();
-        }
+        for (int ks = 0; ks < 4; ++ks) {
+            const int cur = ks & 1, nxt = cur ^ 1;
 #pragma unroll
-        for (int s = 0; s < NM; ++s) {
-            const int i = s / TN, j = s % TN;
-            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bfr[1][j], af[1][i], acc[i][j], 0, 0, 0);
-            // first fragments of k-step t+1 (its stage is complete since the barrier above)
-            if (s < TM) read_a(0, s, 0, st_nxt);
-            else if (s < TM + TN) read_b(0, s - TM, 0, st_nxt);
-            if (s % 3 == 0 && s / 3 < LOADS_PER_TILE / 2) issue_load(t + NSTAGE - 1, stage_ld, LOADS_PER_TILE / 2 + s / 3);
-            KR_SCHED_FENCE();
+            for (int s = 0; s < NM; ++s) {
+                const int i = s / TN, j = s % TN;
+                acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bfr[cur][j], af[cur][i], acc[i][j], 0, 0, 0);
+                if (ks < 3) {
+                    // fragments of the next sub-step, this stage: A blocks next to MFMAs 0..3, B 4..7
+                    if (s < TM) read_a(nxt, s, ks + 1, st_cur);
+                    else if (s < TM + TN) read_b(nxt, s - TM, ks + 1, st_cur);
+                    // the later loads of step t+1
+                    if (ks == 0 && s % 2 == 0) issue_load(t + 1, stage_nxt, kEarly + s / 2);
+                    if (ks == 1 && s % 2 == 0 && s < 4) issue_load(t + 1, stage_nxt, kEarly + 8 + s / 2);
+                } else {
+                    if (s == 3) {
+                        KR_SCHED_FENCE();
+                        __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));
+                        __builtin_amdgcn_s_barrier();
+                    }
+                    // first fragments of k-step t+1
+                    if (s >= 4 && s < 4 + TM) read_a(nxt, s - 4, 0, st_nxt);
+                    else if (s >= 4 + TM && s < 4 + TM + TN) read_b(nxt, s - 4 - TM, 0, st_nxt);
+                    // the first loads of step t+2, into the stage just vacated
+                    if (s >= 4 && s % 2 == 0) issue_load(t + 2, stage_cur, (s - 4) / 2);
+                }
+                KR_SCHED_FENCE();
+            }
         }
     };
-    // Main part: one trip = NSTAGE k-steps, so every LDS stage offset is a compile-time constant
-    // (immediate offsets on the fragment reads, no per-step address arithmetic) and the loop
-    // branch is taken once per NSTAGE steps.  The at most NSTAGE-1 remaining steps follow.
-    static_assert(NSTAGE == 4, "the unrolled trip below spells out four stages");
+    // Main part: one trip = two k-steps, so every LDS stage offset is a compile-time constant
+    // (immediate offsets on the fragment reads) and the loop branch is taken once per 128 MFMAs;
+    // an odd last step follows.
     int t = 0;
 #pragma nounroll
-    for (; t + NSTAGE <= kt_total; t += NSTAGE) {
+    for (; t + 2 <= kt_total; t += 2) {
         k_step(t, std::integral_constant<uint32_t, 0>{});
         k_step(t + 1, std::integral_constant<uint32_t, 1>{});
-        k_step(t + 2, std::integral_constant<uint32_t, 2>{});
-        k_step(t + 3, std::integral_constant<uint32_t, 3>{});
     }
     pin_accumulators();
-    {
-        uint32_t stage_cur = 0;   // t is a multiple of NSTAGE here
-#pragma nounroll
-        for (; t < kt_total; ++t) {
-            k_step(t, stage_cur);
-            stage_cur = stage_cur + 1 == NSTAGE ? 0 : stage_cur + 1;
-        }
-    }
+    if (t < kt_total) k_step(t, std::integral_constant<uint32_t, 0>{});
     // drain the tail's surplus loads before the LDS is reused
     __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));
     __syncthreads();
@@ -417,7 +418,7 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_dtl_kernel(const GemmArgs g)
 }  // namespace
 
 bool gemm_dtl_supported(const GemmArgs& g) {
-    return g.M % BM == 0 && g.N % BN == 0 && g.K % BKD == 0 && g.K >= (NSTAGE - 1) * BKD &&
+    return g.M % BM == 0 && g.N % BN == 0 && g.K % BKD == 0 && g.K >= BKD &&
            (int64_t)BM * g.lda * 2 < 0x7fffffffLL && (int64_t)(BN > 64 ? BN : 64) * g.ldb * 2 < 0x7fffffffLL;
 }
 
