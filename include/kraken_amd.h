@@ -3,8 +3,10 @@
  *
  * The local (one-rank) arithmetic of Kraken's fused communication+compute
  * kernels, written for AMD MI355X (gfx950).  The W peer symmetric-memory
- * buffers of the reference are replaced by W slices of one device tensor
- * ("stack"): slice r starts at  stack + r * slice_stride  elements.
+ * buffers of the reference are W buffers on this GPU, given in one of two
+ * forms: as the W slices of one device tensor ("stack": slice r starts at
+ * stack + r * slice_stride  elements), or, in the kr_*_ptrs_bf16 entry
+ * points, as a table of W device pointers to separate allocations.
  *
  * Conventions for every entry point
  *   - all data pointers are DEVICE pointers; bf16 = 2-byte bfloat16;
@@ -157,6 +159,51 @@ int kr_gemm_reduce_bf16(const void* A, int64_t lda_m, int64_t lda_k,
                         int64_t band_row0, int64_t band_rows,
                         void* c_full, void* out, int out_is_fp32,
                         int64_t tile_pivot, void* stream);
+
+/*
+ * Pointer-table forms.  `bufs` (`peers` for the GEMM) is a HOST array of W
+ * (n_peers) device pointers, one buffer per rank, each 16-byte aligned and at
+ * least as long as the stacked form's slice would be; it is copied into the
+ * launch, so the array may be reused as soon as the call returns.  Everything
+ * else -- arithmetic, order of the adds, requirements, error codes -- is that
+ * of the stacked entry point of the same name, whose kernels these share
+ * (results are bit-identical for equal inputs).
+ *
+ * They replace the same reference kernels as their stacked forms, at the
+ * interface those kernels actually have -- one buffer per rank, handed over
+ * either as a tuple of W tensors from `symm_mem_hdl.get_buffer(i, ...)`
+ *   kraken/comm/one_shot_all_reduce.py:93-97,103        (read at :44)
+ *   kraken/fused/gemm_one_shot_all_reduce_fused.py:141-146,157 (read at :86-91)
+ *   kraken/fused/gemm_reduce_scatter_fused.py:196-201,212      (read at :120)
+ * or as the device table `symm_mem_hdl.buffer_ptrs_dev`, read by
+ * `tl.load(buffer_ptrs + i)`
+ *   kraken/comm/two_shot_all_reduce.py:141              (read at :59)
+ *   kraken/fused/one_shot_all_reduce_bias.py:158        (read at :88)
+ *   kraken/fused/two_shot_all_reduce_bias.py:175        (read at :74)
+ *   kraken/fused/one_shot_all_reduce_bias_rms_norm.py:150     (read at :78)
+ *   kraken/fused/two_shot_all_reduce_bias_rms_norm.py:202     (read at :89).
+ * A binding that holds the rendezvous handle passes the data pointers of its
+ * W buffers; the local rank's buffer is one of the W entries for the reduces
+ * and is left out (n_peers = W - 1, each entry moved on to the band's first
+ * row) for the GEMM.
+ */
+int kr_reduce_ptrs_bf16(const void* const* bufs, int W, int64_t numel,
+                        const void* bias, int64_t bias_numel, int64_t D, int bias_first,
+                        void* out, void* stream);
+int kr_reduce_striped_ptrs_bf16(const void* const* bufs, int W, int64_t numel,
+                                const void* bias, int64_t stripe_block, int rank,
+                                void* out, void* stream);
+int kr_reduce_rmsnorm_ptrs_bf16(const void* const* bufs, int W, int64_t rows, int64_t D,
+                                const void* bias, int bias_is_vector, const void* w, float eps,
+                                void* y, void* stream);
+int kr_gemm_reduce_ptrs_bf16(const void* A, int64_t lda_m, int64_t lda_k,
+                             const void* B, int64_t ldb_k, int64_t ldb_n,
+                             int64_t M, int64_t N, int64_t K,
+                             const void* const* peers, int n_peers,
+                             const void* bias,
+                             int64_t band_row0, int64_t band_rows,
+                             void* c_full, void* out, int out_is_fp32,
+                             int64_t tile_pivot, void* stream);
 
 /*
  * Tile reduce of the copy-engine reduce-scatter variant: `in` is [W*rows, N]

@@ -29,6 +29,23 @@ _SIGNATURES = {
         c_int,
         [c_void_p, c_int, c_int64, c_int64, c_void_p, c_int64, c_int64, c_int, c_void_p, c_void_p],
     ),
+    "kr_reduce_ptrs_bf16": (
+        c_int,
+        [c_void_p, c_int, c_int64, c_void_p, c_int64, c_int64, c_int, c_void_p, c_void_p],
+    ),
+    "kr_reduce_striped_ptrs_bf16": (
+        c_int,
+        [c_void_p, c_int, c_int64, c_void_p, c_int64, c_int, c_void_p, c_void_p],
+    ),
+    "kr_reduce_rmsnorm_ptrs_bf16": (
+        c_int,
+        [c_void_p, c_int, c_int64, c_int64, c_void_p, c_int, c_void_p, c_float, c_void_p, c_void_p],
+    ),
+    "kr_gemm_reduce_ptrs_bf16": (
+        c_int,
+        [c_void_p, c_int64, c_int64, c_void_p, c_int64, c_int64, c_int64, c_int64, c_int64,
+         c_void_p, c_int, c_void_p, c_int64, c_int64, c_void_p, c_void_p, c_int, c_int64, c_void_p],
+    ),
     "kr_reduce_striped_bf16": (
         c_int,
         [c_void_p, c_int, c_int64, c_int64, c_void_p, c_int64, c_int, c_void_p, c_void_p],

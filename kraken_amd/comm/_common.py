@@ -1,37 +1,109 @@
 """Shared argument handling of the W-way reduce wrappers."""
 from __future__ import annotations
 
+import ctypes
+from typing import Sequence
+
 import torch
 
 from .. import _lib
 
 
-def check_stack(stacked: torch.Tensor) -> tuple[int, int, int]:
-    """Validate a ``[W, ...]`` stack; return (W, slice_capacity, slice_stride) in elements.
+class PeerBuffers:
+    """The W buffers a reduce reads: one per rank, all on this GPU.
+
+    Stands in for the peers' symmetric-memory buffers of the reference
+    (``symm_mem_hdl.buffer_ptrs_dev``, ``kraken/comm/one_shot_all_reduce.py:96-99``).
+    Two forms are accepted wherever the reference takes its symmetric buffer:
+
+    * one ``[W, ...]`` tensor whose slices are the W buffers (slices must be
+      contiguous, the stride between them is free) — goes to the stacked entry
+      points of the library;
+    * a list or tuple of W separately allocated tensors of one shape — goes to
+      the pointer-table entry points (``kr_*_ptrs_bf16``), which is also how W
+      real peer mappings would be handed over.
+
+    Both forms give bit-identical results: the kernels are the same.
+    """
+
+    def __init__(self, buffers: torch.Tensor | Sequence[torch.Tensor]):
+        if isinstance(buffers, torch.Tensor):
+            assert buffers.dim() >= 2, "expected a stacked tensor of shape [W, ...]"
+            assert buffers.dtype == torch.bfloat16, "Only bfloat16 is supported for now."
+            self.W = buffers.shape[0]
+            assert self.W >= 1
+            assert buffers[0].is_contiguous(), "each of the W slices must be contiguous"
+            self.cap = buffers[0].numel()
+            self.stride = buffers.stride(0) if self.W > 1 else self.cap
+            self.stacked = buffers
+            self.tensors = [buffers]
+        else:
+            bufs = list(buffers)
+            assert len(bufs) >= 1, "expected W >= 1 buffers"
+            for t in bufs:
+                assert isinstance(t, torch.Tensor), "expected a tensor or a sequence of tensors"
+                assert t.dtype == torch.bfloat16, "Only bfloat16 is supported for now."
+                assert t.is_contiguous(), "each of the W buffers must be contiguous"
+                assert t.shape == bufs[0].shape, "the W buffers must have one shape"
+            self.W = len(bufs)
+            self.cap = bufs[0].numel()
+            self.stride = None
+            self.stacked = None
+            self.tensors = bufs
+
+    def slice(self, rank: int) -> torch.Tensor:
+        """Buffer of rank ``rank``."""
+        return self.stacked[rank] if self.stacked is not None else self.tensors[rank]
+
+    def _table(self, elem_off: int):
+        # host array of W device pointers, each moved on by elem_off bf16 elements
+        return (ctypes.c_void_p * self.W)(*[t.data_ptr() + 2 * elem_off for t in self.tensors])
+
+    def reduce(self, elem_off, numel, bias_ptr, bias_numel, D, bias_first, out_ptr, stream) -> int:
+        """``kr_reduce_bf16`` / ``kr_reduce_ptrs_bf16`` on elements [elem_off, elem_off + numel)."""
+        lib = _lib.load()
+        if self.stacked is not None:
+            return lib.kr_reduce_bf16(self.stacked.data_ptr() + 2 * elem_off, self.W, self.stride, numel,
+                                      bias_ptr, bias_numel, D, bias_first, out_ptr, stream)
+        return lib.kr_reduce_ptrs_bf16(self._table(elem_off), self.W, numel, bias_ptr, bias_numel, D,
+                                       bias_first, out_ptr, stream)
+
+    def reduce_striped(self, numel, bias_ptr, block, rank, out_ptr, stream) -> int:
+        lib = _lib.load()
+        if self.stacked is not None:
+            return lib.kr_reduce_striped_bf16(self.stacked.data_ptr(), self.W, self.stride, numel, bias_ptr,
+                                              block, rank, out_ptr, stream)
+        return lib.kr_reduce_striped_ptrs_bf16(self._table(0), self.W, numel, bias_ptr, block, rank, out_ptr,
+                                               stream)
+
+    def reduce_rmsnorm(self, rows, D, bias_ptr, bias_is_vector, w_ptr, eps, y_ptr, stream) -> int:
+        lib = _lib.load()
+        if self.stacked is not None:
+            return lib.kr_reduce_rmsnorm_bf16(self.stacked.data_ptr(), self.W, self.stride, rows, D, bias_ptr,
+                                              bias_is_vector, w_ptr, eps, y_ptr, stream)
+        return lib.kr_reduce_rmsnorm_ptrs_bf16(self._table(0), self.W, rows, D, bias_ptr, bias_is_vector,
+                                               w_ptr, eps, y_ptr, stream)
+
+
+def check_stack(stacked: torch.Tensor | Sequence[torch.Tensor]) -> PeerBuffers:
+    """Validate the W buffers (stacked tensor or sequence of tensors).
 
     Mirrors the dtype/alignment asserts of ``kraken/comm/one_shot_all_reduce.py:79-80``.
     """
-    assert stacked.dim() >= 2, "expected a stacked tensor of shape [W, ...]"
-    assert stacked.dtype == torch.bfloat16, "Only bfloat16 is supported for now."
-    W = stacked.shape[0]
-    assert W >= 1
-    assert stacked[0].is_contiguous(), "each of the W slices must be contiguous"
-    cap = stacked[0].numel()
-    stride = stacked.stride(0) if W > 1 else cap
-    return W, cap, stride
+    return PeerBuffers(stacked)
 
 
-def stage_input(stacked: torch.Tensor, input_tensor: torch.Tensor | None, rank: int) -> None:
-    """Copy ``input_tensor`` into slice ``rank`` of the stack.
+def stage_input(peers: PeerBuffers, input_tensor: torch.Tensor | None, rank: int) -> None:
+    """Copy ``input_tensor`` into the buffer of rank ``rank``.
 
     Stands in for the copy-in stage of the reference kernels
     (``kraken/fused/one_shot_all_reduce_bias.py:56-65``).  Skipped when the
-    tensor already is (a prefix of) that slice.
+    tensor already is (a prefix of) that buffer.
     """
     if input_tensor is None:
         return
     n = input_tensor.numel()
-    dst = stacked[rank].reshape(-1)[:n]
+    dst = peers.slice(rank).reshape(-1)[:n]
     if dst.data_ptr() == input_tensor.data_ptr():
         return
     dst.copy_(input_tensor.reshape(-1))

@@ -7,12 +7,12 @@ from .. import _lib
 from ._common import check_stack
 
 
-def _share_rows(tensor: torch.Tensor, rank: int, W: int) -> tuple[int, int, tuple[int, ...]]:
-    """Contiguous 1/W chunk of a slice: (offset, numel, shape)."""
-    numel = tensor[0].numel()
+def _share_rows(one: torch.Tensor, rank: int, W: int) -> tuple[int, int, tuple[int, ...]]:
+    """Contiguous 1/W chunk of a slice ``one``: (offset, numel, shape)."""
+    numel = one.numel()
     assert numel % W == 0, "the number of elements must be divisible by the world size"
     share = numel // W
-    shape = tuple(tensor.shape[1:])
+    shape = tuple(one.shape)
     if len(shape) >= 1 and shape[0] % W == 0:
         out_shape = (shape[0] // W, *shape[1:])
     else:
@@ -20,7 +20,7 @@ def _share_rows(tensor: torch.Tensor, rank: int, W: int) -> tuple[int, int, tupl
     return rank * share, share, out_shape
 
 
-def two_shot_all_reduce(tensor: torch.Tensor, **kwargs) -> torch.Tensor:
+def two_shot_all_reduce(tensor, **kwargs) -> torch.Tensor:
     """Reduce the 1/W share that rank ``rank`` owns in a two-shot all-reduce.
 
     Counterpart of ``kraken.comm.two_shot_all_reduce``
@@ -38,38 +38,36 @@ def two_shot_all_reduce(tensor: torch.Tensor, **kwargs) -> torch.Tensor:
       ``BLOCK_SIZE*W`` elements (``:54,146``), returned compactly as 1-D.
     * ``BLOCK_SIZE`` (default 2048): stripe block for ``layout="striped"``.
 
+    ``tensor`` is the ``[W, ...]`` stack or a list of W separate tensors.
     ``max_num_blocks`` and ``num_warps`` are accepted and ignored.
     """
-    W, numel, stride = check_stack(tensor)
+    peers = check_stack(tensor)
+    W, numel = peers.W, peers.cap
     assert numel % 8 == 0, "The number of elements must be 128-bit aligned."
     rank = kwargs.get("rank", 0)
     layout = kwargs.get("layout", "rows")
     block = kwargs.get("BLOCK_SIZE", 2048)
     assert block % W == 0, "BLOCK_SIZE must be divisible by world_size for two-shot all-reduce"
     assert layout in ("rows", "striped")
-    dev = _lib.require_device(tensor)
+    dev = _lib.require_device(*peers.tensors)
     lib = _lib.load()
     stream = _lib.current_stream(dev)
     if rank is None:
-        out = torch.empty(tensor.shape[1:], dtype=tensor.dtype, device=dev)
-        rc = lib.kr_reduce_bf16(tensor.data_ptr(), W, stride, numel, None, 0, 0, 0, out.data_ptr(), stream)
+        out = torch.empty(peers.slice(0).shape, dtype=torch.bfloat16, device=dev)
+        rc = peers.reduce(0, numel, None, 0, 0, 0, out.data_ptr(), stream)
         _lib.check(rc, "two_shot_all_reduce")
         return out
     assert 0 <= rank < W
     if layout == "striped":
         share = lib.kr_striped_share_numel(numel, W, block, rank)
         _lib.check(min(share, 0), "two_shot_all_reduce")
-        out = torch.empty((share,), dtype=tensor.dtype, device=dev)
-        rc = lib.kr_reduce_striped_bf16(
-            tensor.data_ptr(), W, stride, numel, None, block, rank, out.data_ptr(), stream
-        )
+        out = torch.empty((share,), dtype=torch.bfloat16, device=dev)
+        rc = peers.reduce_striped(numel, None, block, rank, out.data_ptr(), stream)
         _lib.check(rc, "two_shot_all_reduce")
         return out
-    off, share, out_shape = _share_rows(tensor, rank, W)
+    off, share, out_shape = _share_rows(peers.slice(0), rank, W)
     assert share % 8 == 0, "each rank's share must be 128-bit aligned"
-    out = torch.empty(out_shape, dtype=tensor.dtype, device=dev)
-    rc = lib.kr_reduce_bf16(
-        tensor.data_ptr() + 2 * off, W, stride, share, None, 0, 0, 0, out.data_ptr(), stream
-    )
+    out = torch.empty(out_shape, dtype=torch.bfloat16, device=dev)
+    rc = peers.reduce(off, share, None, 0, 0, 0, out.data_ptr(), stream)
     _lib.check(rc, "two_shot_all_reduce")
     return out

@@ -67,6 +67,15 @@ __device__ __forceinline__ u32x4 pack8(const float (&f)[8]) {
 __device__ __forceinline__ u32x4 ld_stream(const u32x4* p) { return __builtin_nontemporal_load(p); }
 __device__ __forceinline__ void st_stream(u32x4* p, u32x4 v) { __builtin_nontemporal_store(v, p); }
 
+// Streaming 128-bit load through a buffer descriptor: the address is the descriptor's base
+// (uniform, in scalar registers) + a 32-bit byte offset per lane, so loads from many
+// buffers share one offset register.  Bytes at or past `bytes` read as zero.
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t stream_rsrc(const void* base, uint32_t bytes) {
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, (int)bytes, 0x00020000);
+}
+__device__ __forceinline__ u32x4 ld_stream(__amdgpu_buffer_rsrc_t rs, uint32_t byte_off) {
+    return __builtin_amdgcn_raw_buffer_load_b128(rs, (int)byte_off, 0, 2 /* non-temporal */);
+}
 // ---- wave64 sum -------------------------------------------------------------
 // Sum over the 64 lanes of a wavefront; every lane returns the total.  The
 // first four steps stay inside a row of 16 lanes and use DPP lane permutes
@@ -89,7 +98,44 @@ __device__ __forceinline__ float wave_sum(float v) {
     return (r0 + r1) + (r2 + r3);
 }
 
+// ---- peer buffers ------------------------------------------------------------
+// The W buffers a reduce reads, one device pointer per rank, passed to the kernels by
+// value (kernel-argument memory, read through scalar loads): the pointer-table entry points
+// copy the caller's table into it.
+struct PeerTab {
+    const u32x4* p[KR_MAX_WORLD];
+    static constexpr bool kTable = true;
+    __device__ __forceinline__ const u32x4* at(int r) const { return p[r]; }
+};
+// The same interface for the W slices of one stacked tensor, stride_v 128-bit vectors apart:
+// the kernels are instantiated for both, so each form keeps its own address arithmetic.
+struct StackedPeers {
+    const u32x4* base;
+    int64_t stride_v;
+    static constexpr bool kTable = false;
+    __device__ __forceinline__ const u32x4* at(int r) const { return base + r * stride_v; }
+};
+
 // ---- host-side checks -------------------------------------------------------
 static inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+// Table of the W slices of a stacked tensor (slice r at stack + r * stride elements of bf16).
+// Entries past W repeat entry 0, so every entry can be dereferenced.
+static inline void peer_tab_stacked(PeerTab& t, const void* stack, int W, int64_t stride_elems) {
+    const uint16_t* b = static_cast<const uint16_t*>(stack);
+    for (int r = 0; r < KR_MAX_WORLD; ++r)
+        t.p[r] = reinterpret_cast<const u32x4*>(r < W ? b + (int64_t)r * stride_elems : b);
+}
+
+// Table copied from a caller's host array of W device pointers; KR_OK or the argument error.
+static inline int peer_tab_from_ptrs(PeerTab& t, const void* const* bufs, int W) {
+    if (bufs == nullptr) return KR_ERR_NULL_POINTER;
+    for (int r = 0; r < W; ++r) {
+        if (bufs[r] == nullptr) return KR_ERR_NULL_POINTER;
+        if (!aligned16(bufs[r])) return KR_ERR_ALIGNMENT;
+    }
+    for (int r = 0; r < KR_MAX_WORLD; ++r) t.p[r] = static_cast<const u32x4*>(bufs[r < W ? r : 0]);
+    return KR_OK;
+}
 
 }  // namespace kr

@@ -331,7 +331,7 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_reduce_kernel(const GemmArgs
     // LDS is reused by the epilogue
     __syncthreads();
 
-    gemm_epilogue<BM, WTM, WTN, TM, TN, EVEN, EP_WAVE>(g, acc, smem, m0, n0, wm, wn, lane, wave);
+    gemm_epilogue<BM, WTM, WTN, TM, TN, EVEN, EP_WAVE>(g, g.n_peers, g.bias, acc, smem, m0, n0, wm, wn, lane, wave);
 }
 
 template <int BM, int BN, int WM, int WN>
@@ -364,11 +364,13 @@ static hipError_t launch_gemm(const GemmArgs& g, bool b_nt, bool even, hipStream
 
 using namespace kr;
 
-extern "C" int kr_gemm_reduce_bf16(const void* A, int64_t lda_m, int64_t lda_k, const void* B, int64_t ldb_k,
-                                   int64_t ldb_n, int64_t M, int64_t N, int64_t K, const void* peers,
-                                   int n_peers, int64_t peers_stride, const void* bias, int64_t band_row0,
-                                   int64_t band_rows, void* c_full, void* out, int out_is_fp32,
-                                   int64_t tile_pivot, void* stream) {
+// Everything of the two entry points except the peers: argument checks in the documented
+// order, then tile choice and launch.  `peers_given` is the stacked base or the table.
+static int gemm_reduce(const void* A, int64_t lda_m, int64_t lda_k, const void* B, int64_t ldb_k, int64_t ldb_n,
+                       int64_t M, int64_t N, int64_t K, const void* peers_given, int n_peers,
+                       const void* const* peer_ptrs, int64_t peers_stride, const void* bias,
+                       int64_t band_row0, int64_t band_rows, void* c_full, void* out, int out_is_fp32,
+                       int64_t tile_pivot, void* stream) {
     if (M < 0 || N < 0 || K < 0 || M > 0x7fffffffLL || N > 0x7fffffffLL || K > 0x7fffffffLL)
         return KR_ERR_BAD_DIM;
     if (n_peers < 0 || n_peers >= KR_MAX_WORLD) return KR_ERR_WORLD_SIZE;
@@ -378,27 +380,33 @@ extern "C" int kr_gemm_reduce_bf16(const void* A, int64_t lda_m, int64_t lda_k, 
     if (K == 0) return KR_ERR_BAD_DIM;
     if (A == nullptr || B == nullptr) return KR_ERR_NULL_POINTER;
     if (band_rows > 0 && out == nullptr) return KR_ERR_NULL_POINTER;
-    if (n_peers > 0 && peers == nullptr) return KR_ERR_NULL_POINTER;
+    if (n_peers > 0 && peers_given == nullptr) return KR_ERR_NULL_POINTER;
     if (lda_k != 1) return KR_ERR_LAYOUT;
     const bool b_nt = (ldb_k == 1 && (ldb_n != 1 || N == 1));
     if (!b_nt && ldb_n != 1) return KR_ERR_LAYOUT;
     const int64_t ldb = b_nt ? ldb_n : ldb_k;
     if (lda_m < K || (b_nt ? ldb < K : ldb < N)) return KR_ERR_LAYOUT;
-    if (lda_m % 8 != 0 || ldb % 8 != 0 || peers_stride % 8 != 0) return KR_ERR_ALIGNMENT;
-    if (!aligned16(A) || !aligned16(B) || !aligned16(peers) || !aligned16(bias) || !aligned16(c_full) ||
-        !aligned16(out))
+    if (lda_m % 8 != 0 || ldb % 8 != 0) return KR_ERR_ALIGNMENT;
+    if (!aligned16(A) || !aligned16(B) || !aligned16(bias) || !aligned16(c_full) || !aligned16(out))
         return KR_ERR_ALIGNMENT;
-    if (n_peers > 0 && peers_stride < band_rows * N) return KR_ERR_BAD_DIM;
 
     GemmArgs g;
+    if (peer_ptrs != nullptr) {
+        // separate allocations: a table of n_peers device pointers
+        const int rc = n_peers > 0 ? peer_tab_from_ptrs(g.peer, peer_ptrs, n_peers) : KR_OK;
+        if (rc != KR_OK) return rc;
+        if (n_peers == 0) peer_tab_stacked(g.peer, A, 0, 0);
+    } else {
+        if (peers_stride % 8 != 0 || !aligned16(peers_given)) return KR_ERR_ALIGNMENT;
+        if (n_peers > 0 && peers_stride < band_rows * N) return KR_ERR_BAD_DIM;
+        peer_tab_stacked(g.peer, n_peers > 0 ? peers_given : A, n_peers, peers_stride);
+    }
     g.A = (const uint16_t*)A;
     g.B = (const uint16_t*)B;
     g.lda = lda_m;
     g.ldb = ldb;
     g.M = (int)M; g.N = (int)N; g.K = (int)K;
-    g.peers = (const uint16_t*)peers;
     g.n_peers = n_peers;
-    g.peers_stride = peers_stride;
     g.bias = (const uint16_t*)bias;
     g.band_row0 = (int)band_row0;
     g.band_rows = (int)band_rows;
@@ -440,4 +448,25 @@ extern "C" int kr_gemm_reduce_bf16(const void* A, int64_t lda_m, int64_t lda_k, 
     hipError_t e = dtl ? launch_gemm_dtl(g, b_nt, (hipStream_t)stream)
                        : launch_gemm<128, 128, 2, 2>(g, b_nt, even, (hipStream_t)stream);
     return (int)e;
+}
+
+extern "C" int kr_gemm_reduce_bf16(const void* A, int64_t lda_m, int64_t lda_k, const void* B, int64_t ldb_k,
+                                   int64_t ldb_n, int64_t M, int64_t N, int64_t K, const void* peers,
+                                   int n_peers, int64_t peers_stride, const void* bias, int64_t band_row0,
+                                   int64_t band_rows, void* c_full, void* out, int out_is_fp32,
+                                   int64_t tile_pivot, void* stream) {
+    return gemm_reduce(A, lda_m, lda_k, B, ldb_k, ldb_n, M, N, K, peers, n_peers, nullptr, peers_stride, bias,
+                       band_row0, band_rows, c_full, out, out_is_fp32, tile_pivot, stream);
+}
+
+extern "C" int kr_gemm_reduce_ptrs_bf16(const void* A, int64_t lda_m, int64_t lda_k, const void* B,
+                                        int64_t ldb_k, int64_t ldb_n, int64_t M, int64_t N, int64_t K,
+                                        const void* const* peers, int n_peers, const void* bias,
+                                        int64_t band_row0, int64_t band_rows, void* c_full, void* out,
+                                        int out_is_fp32, int64_t tile_pivot, void* stream) {
+    // an empty table with n_peers == 0 is a plain GEMM; the flag below still selects the table path
+    static const void* const kNoPeers[1] = {nullptr};
+    return gemm_reduce(A, lda_m, lda_k, B, ldb_k, ldb_n, M, N, K, peers, n_peers,
+                       peers != nullptr ? peers : kNoPeers, 0, bias, band_row0, band_rows, c_full, out,
+                       out_is_fp32, tile_pivot, stream);
 }

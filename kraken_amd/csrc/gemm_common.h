@@ -13,9 +13,8 @@ struct GemmArgs {
     int64_t lda;   // elements between rows of A (k is contiguous)
     int64_t ldb;   // NT: elements between n-rows of B^T; NN: elements between k-rows of B
     int M, N, K;
-    const uint16_t* peers;
+    PeerTab peer;        // peer.p[j]: partial sums of peer j, [band_rows, N] bf16 (j < n_peers)
     int n_peers;
-    int64_t peers_stride;
     const uint16_t* bias;
     int band_row0, band_rows;
     uint16_t* c_full;
@@ -73,7 +72,8 @@ __device__ __forceinline__ void tile_schedule(const GemmArgs& g, int& tile_m_out
 // F32 = true (fp32 result: the reference's fused all-reduce keeps fp32 from the accumulator to
 // the output, kraken/fused/gemm_one_shot_all_reduce_fused.py:65-99): the patch holds fp32.
 template <bool F32, int BM, int WTM, int WTN, int TM, int TN, bool EVEN, int EP_WAVE>
-__device__ __forceinline__ void gemm_epilogue_impl(const GemmArgs& g, const f32x16 (&acc)[TM][TN], unsigned char* smem,
+__device__ __forceinline__ void gemm_epilogue_impl(const GemmArgs& g, const int n_peers, const uint16_t* bias,
+                                                   const f32x16 (&acc)[TM][TN], unsigned char* smem,
                                                    int m0, int n0, int wm, int wn, int lane, int wave) {
     // After the barrier above no wave reads the pipeline stages any more, and from here on
     // every wave touches only its own LDS patch, so no further workgroup barrier is needed
@@ -102,8 +102,8 @@ __device__ __forceinline__ void gemm_epilogue_impl(const GemmArgs& g, const f32x
 
     float bias_f[8];
     zero8(bias_f);
-    const bool has_bias = g.bias != nullptr;
-    if (has_bias) add8(*(const u32x4*)(g.bias + (EVEN ? n : min(n, g.N - 8))), bias_f);
+    const bool has_bias = bias != nullptr;
+    if (has_bias) add8(*(const u32x4*)(bias + (EVEN ? n : min(n, g.N - 8))), bias_f);
 
     // Round-to-nearest-even pack of two fp32 to bf16, pinned where it is written: the
     // accumulators do not change inside the slab loop, so an ordinary conversion -- or, for
@@ -187,9 +187,9 @@ __device__ __forceinline__ void gemm_epilogue_impl(const GemmArgs& g, const f32x
         constexpr int kFastBatch = BM >= 256 ? 2 : 1;   // chunks per batch (the small tile keeps two workgroups per CU)
         constexpr int kFastBatches = EP_ITERS / kFastBatch;
         static_assert(kFastBatches % 2 == 0, "the two peer buffers alternate with a static parity");
-        if (EVEN && g.n_peers == kFastPeers && wave_m0 >= band_lo && wave_m0 + WTM <= band_hi) {
+        if (EVEN && n_peers == kFastPeers && wave_m0 >= band_lo && wave_m0 + WTM <= band_hi) {
             u32x4 pv[2][kFastBatch][kFastPeers];
-            const uint16_t* peer_base = g.peers + ((int64_t)(wave_m0 - band_lo + lane_r) * g.N + n);
+            const int64_t peer_off = (int64_t)(wave_m0 - band_lo + lane_r) * g.N + n;
             const int64_t chunk_step = (int64_t)(64 / CPR) * g.N;   // elements between consecutive chunks of a lane
             auto issue = [&](auto buf_c, int chunk_abs) __attribute__((always_inline)) {
                 constexpr int buf = decltype(buf_c)::value;
@@ -198,7 +198,7 @@ __device__ __forceinline__ void gemm_epilogue_impl(const GemmArgs& g, const f32x
 #pragma unroll
                     for (int q = 0; q < kFastPeers; ++q)
                         pv[buf][c][q] =
-                            ld_stream((const u32x4*)(peer_base + q * g.peers_stride + (chunk_abs + c) * chunk_step));
+                            ld_stream((const u32x4*)((const uint16_t*)g.peer.p[q] + peer_off + (chunk_abs + c) * chunk_step));
             };
             issue(std::integral_constant<int, 0>{}, 0);
 #pragma nounroll
@@ -273,21 +273,21 @@ __device__ __forceinline__ void gemm_epilogue_impl(const GemmArgs& g, const f32x
             const int64_t safe_off = min(n, g.N - 8);
 #pragma unroll
             for (int q0 = 0; q0 < KR_MAX_WORLD - 1; q0 += kPeerGroup) {
-                if (q0 < g.n_peers) {
+                if (q0 < n_peers) {
                     u32x4 pv[kChunkBatch][kPeerGroup];
 #pragma unroll
                     for (int c = 0; c < kChunkBatch; ++c)
 #pragma unroll
                         for (int q = 0; q < kPeerGroup; ++q) {
-                            const int qq = min(q0 + q, g.n_peers - 1);
+                            const int qq = min(q0 + q, n_peers - 1);
                             pv[c][q] = ld_stream(
-                                (const u32x4*)(g.peers + qq * g.peers_stride + (in_band[c] ? off[c] : safe_off)));
+                                (const u32x4*)((const uint16_t*)g.peer.p[qq] + (in_band[c] ? off[c] : safe_off)));
                         }
 #pragma unroll
                     for (int c = 0; c < kChunkBatch; ++c)
 #pragma unroll
                         for (int q = 0; q < kPeerGroup; ++q) {
-                            const uint32_t keep = (in_band[c] && q0 + q < g.n_peers) ? 0xffffffffu : 0u;
+                            const uint32_t keep = (in_band[c] && q0 + q < n_peers) ? 0xffffffffu : 0u;
                             add8(u32x4{pv[c][q].x & keep, pv[c][q].y & keep, pv[c][q].z & keep, pv[c][q].w & keep}, f[c]);
                         }
                 }
@@ -315,7 +315,7 @@ __device__ __forceinline__ void gemm_epilogue_impl(const GemmArgs& g, const f32x
         for (int b0 = 0; b0 < EP_ITERS; b0 += kChunkBatch) {
             if (all_out) {
                 slab_batch(std::integral_constant<int, -2>{}, slab_m0, b0);
-            } else if (all_in && g.n_peers == 0) {
+            } else if (all_in && n_peers == 0) {
                 slab_batch(std::integral_constant<int, 0>{}, slab_m0, b0);
             } else {
                 slab_batch(std::integral_constant<int, -1>{}, slab_m0, b0);
@@ -325,11 +325,15 @@ __device__ __forceinline__ void gemm_epilogue_impl(const GemmArgs& g, const f32x
     }
 }
 
+// n_peers and bias are what is still to be added here (a kernel that has already put the
+// peers or the bias into the accumulators passes 0 / nullptr); g is only read, never copied,
+// so the peer table stays in kernel-argument memory.
 template <int BM, int WTM, int WTN, int TM, int TN, bool EVEN, int EP_WAVE>
-__device__ __forceinline__ void gemm_epilogue(const GemmArgs& g, const f32x16 (&acc)[TM][TN], unsigned char* smem,
+__device__ __forceinline__ void gemm_epilogue(const GemmArgs& g, int n_peers, const uint16_t* bias,
+                                              const f32x16 (&acc)[TM][TN], unsigned char* smem,
                                               int m0, int n0, int wm, int wn, int lane, int wave) {
-    if (g.out_is_fp32) gemm_epilogue_impl<true, BM, WTM, WTN, TM, TN, EVEN, EP_WAVE>(g, acc, smem, m0, n0, wm, wn, lane, wave);
-    else gemm_epilogue_impl<false, BM, WTM, WTN, TM, TN, EVEN, EP_WAVE>(g, acc, smem, m0, n0, wm, wn, lane, wave);
+    if (g.out_is_fp32) gemm_epilogue_impl<true, BM, WTM, WTN, TM, TN, EVEN, EP_WAVE>(g, n_peers, bias, acc, smem, m0, n0, wm, wn, lane, wave);
+    else gemm_epilogue_impl<false, BM, WTM, WTN, TM, TN, EVEN, EP_WAVE>(g, n_peers, bias, acc, smem, m0, n0, wm, wn, lane, wave);
 }
 
 }  // namespace kr

@@ -267,13 +267,13 @@ __device__ __forceinline__ void gemm_dtl_tile(const GemmArgs& g, unsigned char* 
             pa[jh] = region + (uint32_t)(row * 256 + (((2 * jh + (lane >> 5)) ^ (row & 15)) << 4));
         }
         const int n_items = g.n_peers * TM;    // item = (peer q, slab i), q-major
-        const uint16_t* wave_base = g.peers + ((int64_t)(m0 + wm * WTM - band_lo) * g.N + n0 + wn * WTN);
+        const int64_t wave_off = (int64_t)(m0 + wm * WTM - band_lo) * g.N + n0 + wn * WTN;
         auto issue_item = [&](int it, int stage) __attribute__((always_inline)) {
             // past the end: all lanes re-read 16 bytes of the last item (the load count per item
             // is fixed for the vmcnt arithmetic; the data is never used)
             const bool live = it < n_items;
             const int itc = min(it, n_items - 1);
-            const i32x4 rs = make_rsrc(wave_base + (int64_t)(itc >> 2) * g.peers_stride + (int64_t)(itc & 3) * 32 * g.N);
+            const i32x4 rs = make_rsrc((const uint16_t*)g.peer.p[itc >> 2] + wave_off + (int64_t)(itc & 3) * 32 * g.N);
 #pragma unroll
             for (int r = 0; r < kItemLoads; ++r)
                 lds_dma_b128_stream(rs, region + stage * kItemBytes + r * 1024, live ? pvoff[r & 3] : 0u,
@@ -398,10 +398,9 @@ __device__ __forceinline__ void gemm_dtl_tile(const GemmArgs& g, unsigned char* 
     pin_accumulators();
     if (!PEERS_FIRST && mfma_peers) peer_phase();
     pin_accumulators();
-    GemmArgs ge = g;
-    if (mfma_peers) ge.n_peers = 0;   // already in the accumulators
-    if (bias_in_acc) ge.bias = nullptr;
-    gemm_epilogue<BM, WTM, WTN, TM, TN, true, EP_WAVE>(ge, acc, smem, m0, n0, wm, wn, lane, wave);
+    // peers and bias that are already in the accumulators are not added again
+    gemm_epilogue<BM, WTM, WTN, TM, TN, true, EP_WAVE>(g, mfma_peers ? 0 : g.n_peers, bias_in_acc ? nullptr : g.bias,
+                                                       acc, smem, m0, n0, wm, wn, lane, wave);
 }
 #undef KR_SCHED_FENCE
 

@@ -1,4 +1,5 @@
-// W-way elementwise reduce (+bias) over the W slices of a stacked bf16 tensor.
+// W-way elementwise reduce (+bias) over W bf16 buffers (the slices of a stacked tensor, or
+// W separate allocations named by a pointer table).
 //
 // HBM-bound: per output vector of 8 elements the kernel reads W*16 B (+16 B of
 // bias) and writes 16 B, i.e. (W+1)*2 bytes per element.  A workgroup walks the
@@ -19,9 +20,9 @@ constexpr int kMaxBlocks = 4 * 256;   // 4 workgroups per CU
 enum BiasMode { kNoBias = 0, kFullBias = 1, kVectorBias = 2 };
 
 // WT > 0: W known at compile time (loop fully unrolled); WT == 0: run-time W.
-template <int WT, int BIAS, bool BIAS_FIRST, int kUnroll>
+template <class SRC, int WT, int BIAS, bool BIAS_FIRST, int kUnroll>
 __global__ __launch_bounds__(kThreads) void reduce_kernel(
-    const u32x4* __restrict__ stack, int w_rt, int64_t slice_stride_v, int64_t nvec,
+    const SRC src, int w_rt, int64_t nvec,
     const u32x4* __restrict__ bias, uint32_t d_vec, u32x4* __restrict__ out) {
     const int W = WT > 0 ? WT : w_rt;
     for (int64_t blk = blockIdx.x; blk * (kThreads * kUnroll) < nvec; blk += gridDim.x) {
@@ -40,11 +41,23 @@ __global__ __launch_bounds__(kThreads) void reduce_kernel(
         }
         if (WT > 0) {
             u32x4 v[WT > 0 ? WT : 1][kUnroll];
+            if constexpr (SRC::kTable) {
+                // separate buffers: each buffer's block through a descriptor (base = buffer +
+                // block, in scalar registers), so all W buffers share one byte offset per (lane, u)
+                constexpr uint32_t kBlockBytes = kThreads * kUnroll * 16;
 #pragma unroll
-            for (int r = 0; r < WT; ++r)
+                for (int r = 0; r < WT; ++r) {
+                    const __amdgpu_buffer_rsrc_t rs = stream_rsrc(src.at(r) + blk * (kThreads * kUnroll), kBlockBytes);
 #pragma unroll
-                for (int u = 0; u < kUnroll; ++u)
-                    v[r][u] = ld_stream(stack + r * slice_stride_v + base + (int64_t)u * kThreads);
+                    for (int u = 0; u < kUnroll; ++u) v[r][u] = ld_stream(rs, (threadIdx.x + u * kThreads) * 16u);
+                }
+            } else {
+#pragma unroll
+                for (int r = 0; r < WT; ++r)
+#pragma unroll
+                    for (int u = 0; u < kUnroll; ++u)
+                        v[r][u] = ld_stream(src.at(r) + base + (int64_t)u * kThreads);
+            }
 #pragma unroll
             for (int u = 0; u < kUnroll; ++u) {
                 if (BIAS != kNoBias && BIAS_FIRST) {
@@ -60,15 +73,15 @@ __global__ __launch_bounds__(kThreads) void reduce_kernel(
         } else {
 #pragma unroll
             for (int u = 0; u < kUnroll; ++u) {
-                const u32x4* p = stack + base + (int64_t)u * kThreads;
+                const int64_t i = base + (int64_t)u * kThreads;
                 if (BIAS != kNoBias && BIAS_FIRST) {
                     unpack8(bv[u], acc[u]);
-                    add8(ld_stream(p), acc[u]);
+                    add8(ld_stream(src.at(0) + i), acc[u]);
                 } else {
                     zero8(acc[u]);
-                    add8(ld_stream(p), acc[u]);
+                    add8(ld_stream(src.at(0) + i), acc[u]);
                 }
-                for (int r = 1; r < W; ++r) add8(ld_stream(p + r * slice_stride_v), acc[u]);
+                for (int r = 1; r < W; ++r) add8(ld_stream(src.at(r) + i), acc[u]);
             }
         }
 #pragma unroll
@@ -84,15 +97,14 @@ __global__ __launch_bounds__(kThreads) void reduce_kernel(
             float acc[8];
             u32x4 bv = {0, 0, 0, 0};
             if (BIAS != kNoBias) bv = BIAS == kFullBias ? bias[i] : bias[mod_vec(i, d_vec)];
-            const u32x4* p = stack + i;
             if (BIAS != kNoBias && BIAS_FIRST) {
                 unpack8(bv, acc);
-                add8(p[0], acc);
+                add8(src.at(0)[i], acc);
             } else {
                 zero8(acc);
-                add8(p[0], acc);
+                add8(src.at(0)[i], acc);
             }
-            for (int r = 1; r < W; ++r) add8(p[r * slice_stride_v], acc);
+            for (int r = 1; r < W; ++r) add8(src.at(r)[i], acc);
             if (BIAS != kNoBias && !BIAS_FIRST) add8(bv, acc);
             out[i] = pack8(acc);
         }
@@ -102,18 +114,18 @@ __global__ __launch_bounds__(kThreads) void reduce_kernel(
 
 // Striped ownership: output vector j (compact) comes from input vector
 //   (j / blk_v) * blk_v * W + rank * blk_v + (j % blk_v).
+template <class SRC>
 __global__ __launch_bounds__(kThreads) void reduce_striped_kernel(
-    const u32x4* __restrict__ stack, int W, int64_t slice_stride_v, int64_t share_nvec,
+    const SRC src, int W, int64_t share_nvec,
     const u32x4* __restrict__ bias, uint32_t blk_v, int rank, u32x4* __restrict__ out) {
     const int64_t j = (int64_t)blockIdx.x * kThreads + threadIdx.x;
     if (j >= share_nvec) return;
     const int64_t stripe = j / blk_v;
     const int64_t i = (stripe * W + rank) * blk_v + (j - stripe * blk_v);
     float acc[8];
-    const u32x4* p = stack + i;
     zero8(acc);
-    add8(ld_stream(p), acc);
-    for (int r = 1; r < W; ++r) add8(ld_stream(p + r * slice_stride_v), acc);
+    add8(ld_stream(src.at(0) + i), acc);
+    for (int r = 1; r < W; ++r) add8(ld_stream(src.at(r) + i), acc);
     if (bias != nullptr) add8(ld_stream(bias + i), acc);
     st_stream(out + j, pack8(acc));
 }
@@ -141,8 +153,8 @@ __global__ __launch_bounds__(kThreads) void reduce_rotated_kernel(
 // for inputs too small to give every CU four such blocks (more, smaller workgroups).
 static int pick_unroll(int64_t nvec) { return nvec >= (int64_t)kMaxBlocks * kThreads * 4 ? 4 : 1; }
 
-template <int WT, int BIAS, bool BF>
-static void launch_reduce3(hipStream_t s, const u32x4* stack, int W, int64_t ssv, int64_t nvec, const u32x4* bias,
+template <class SRC, int WT, int BIAS, bool BF>
+static void launch_reduce3(hipStream_t s, const SRC& tab, int W, int64_t nvec, const u32x4* bias,
                            uint32_t d_vec, u32x4* out) {
     const int unroll = pick_unroll(nvec);
     const int64_t per_block = (int64_t)kThreads * unroll;
@@ -150,34 +162,34 @@ static void launch_reduce3(hipStream_t s, const u32x4* stack, int W, int64_t ssv
     if (blocks > kMaxBlocks) blocks = kMaxBlocks;
     const dim3 grid((unsigned)blocks);
     if (unroll == 4)
-        hipLaunchKernelGGL((reduce_kernel<WT, BIAS, BF, 4>), grid, dim3(kThreads), 0, s, stack, W, ssv, nvec, bias,
+        hipLaunchKernelGGL((reduce_kernel<SRC, WT, BIAS, BF, 4>), grid, dim3(kThreads), 0, s, tab, W, nvec, bias,
                            d_vec, out);
     else
-        hipLaunchKernelGGL((reduce_kernel<WT, BIAS, BF, 1>), grid, dim3(kThreads), 0, s, stack, W, ssv, nvec, bias,
+        hipLaunchKernelGGL((reduce_kernel<SRC, WT, BIAS, BF, 1>), grid, dim3(kThreads), 0, s, tab, W, nvec, bias,
                            d_vec, out);
 }
 
-template <int WT, int BIAS>
-static hipError_t launch_reduce2(bool bias_first, hipStream_t s, const u32x4* stack, int W, int64_t ssv,
+template <class SRC, int WT, int BIAS>
+static hipError_t launch_reduce2(bool bias_first, hipStream_t s, const SRC& tab, int W,
                                  int64_t nvec, const u32x4* bias, uint32_t d_vec, u32x4* out) {
     if (bias_first)
-        launch_reduce3<WT, BIAS, true>(s, stack, W, ssv, nvec, bias, d_vec, out);
+        launch_reduce3<SRC, WT, BIAS, true>(s, tab, W, nvec, bias, d_vec, out);
     else
-        launch_reduce3<WT, BIAS, false>(s, stack, W, ssv, nvec, bias, d_vec, out);
+        launch_reduce3<SRC, WT, BIAS, false>(s, tab, W, nvec, bias, d_vec, out);
     return hipGetLastError();
 }
 
-template <int WT>
-static hipError_t launch_reduce1(int mode, bool bias_first, hipStream_t s, const u32x4* stack, int W,
-                                 int64_t ssv, int64_t nvec, const u32x4* bias, uint32_t d_vec, u32x4* out) {
+template <class SRC, int WT>
+static hipError_t launch_reduce1(int mode, bool bias_first, hipStream_t s, const SRC& tab, int W,
+                                 int64_t nvec, const u32x4* bias, uint32_t d_vec, u32x4* out) {
     switch (mode) {
         case kNoBias:
             // without a bias both orders are the same kernel
-            return launch_reduce2<WT, kNoBias>(true, s, stack, W, ssv, nvec, bias, d_vec, out);
+            return launch_reduce2<SRC, WT, kNoBias>(true, s, tab, W, nvec, bias, d_vec, out);
         case kFullBias:
-            return launch_reduce2<WT, kFullBias>(bias_first, s, stack, W, ssv, nvec, bias, d_vec, out);
+            return launch_reduce2<SRC, WT, kFullBias>(bias_first, s, tab, W, nvec, bias, d_vec, out);
         default:
-            return launch_reduce2<WT, kVectorBias>(bias_first, s, stack, W, ssv, nvec, bias, d_vec, out);
+            return launch_reduce2<SRC, WT, kVectorBias>(bias_first, s, tab, W, nvec, bias, d_vec, out);
     }
 }
 
@@ -185,48 +197,73 @@ static hipError_t launch_reduce1(int mode, bool bias_first, hipStream_t s, const
 
 using namespace kr;
 
-static int check_reduce_common(const void* stack, int W, int64_t slice_stride, int64_t numel, const void* out) {
+// Argument checks shared by the stacked and the pointer-table entry points; `first` is the
+// stacked tensor, or the table itself.  Returns KR_OK also for numel == 0.
+static int check_reduce_common(const void* first, int W, int64_t numel, const void* out) {
     if (W < 1 || W > KR_MAX_WORLD) return KR_ERR_WORLD_SIZE;
     if (numel < 0) return KR_ERR_BAD_DIM;
     if (numel % 8 != 0) return KR_ERR_NUMEL_MOD8;
     if (numel == 0) return KR_OK;
-    if (stack == nullptr || out == nullptr) return KR_ERR_NULL_POINTER;
-    if (!aligned16(stack) || !aligned16(out) || slice_stride % 8 != 0) return KR_ERR_ALIGNMENT;
+    if (first == nullptr || out == nullptr) return KR_ERR_NULL_POINTER;
+    if (!aligned16(out)) return KR_ERR_ALIGNMENT;
+    return KR_OK;
+}
+
+static int check_stack(const void* stack, int64_t slice_stride) {
+    if (!aligned16(stack) || slice_stride % 8 != 0) return KR_ERR_ALIGNMENT;
     if (slice_stride < 0) return KR_ERR_BAD_DIM;
     return KR_OK;
 }
 
-extern "C" int kr_reduce_bf16(const void* stack, int W, int64_t slice_stride, int64_t numel, const void* bias,
-                              int64_t bias_numel, int64_t D, int bias_first, void* out, void* stream) {
-    int rc = check_reduce_common(stack, W, slice_stride, numel, out);
-    if (rc != KR_OK) return rc;
-    int mode = kNoBias;
-    if (bias != nullptr) {
-        if (!aligned16(bias)) return KR_ERR_ALIGNMENT;
-        if (bias_numel == numel) {
-            mode = kFullBias;
-        } else if (D > 0 && bias_numel == D && D % 8 == 0 && numel % D == 0) {
-            mode = kVectorBias;
-        } else {
-            return KR_ERR_BIAS_SHAPE;
-        }
-    }
-    if (numel == 0) return KR_OK;
+// bias mode from the bias arguments, or a negative argument error
+static int reduce_bias_mode(const void* bias, int64_t bias_numel, int64_t numel, int64_t D) {
+    if (bias == nullptr) return kNoBias;
+    if (!aligned16(bias)) return KR_ERR_ALIGNMENT;
+    if (bias_numel == numel) return kFullBias;
+    if (D > 0 && bias_numel == D && D % 8 == 0 && numel % D == 0) return kVectorBias;
+    return KR_ERR_BIAS_SHAPE;
+}
+
+template <class SRC>
+static int launch_reduce(const SRC& tab, int W, int64_t numel, const void* bias, int mode, int64_t D,
+                         int bias_first, void* out, void* stream) {
     const int64_t nvec = numel / 8;
     const hipStream_t s = (hipStream_t)stream;
-    const u32x4* sp = (const u32x4*)stack;
     const u32x4* bp = (const u32x4*)bias;
     u32x4* op = (u32x4*)out;
-    const int64_t ssv = slice_stride / 8;
     const uint32_t d_vec = mode == kVectorBias ? (uint32_t)(D / 8) : 1u;
     hipError_t e;
     switch (W) {
-        case 2: e = launch_reduce1<2>(mode, bias_first != 0, s, sp, W, ssv, nvec, bp, d_vec, op); break;
-        case 4: e = launch_reduce1<4>(mode, bias_first != 0, s, sp, W, ssv, nvec, bp, d_vec, op); break;
-        case 8: e = launch_reduce1<8>(mode, bias_first != 0, s, sp, W, ssv, nvec, bp, d_vec, op); break;
-        default: e = launch_reduce1<0>(mode, bias_first != 0, s, sp, W, ssv, nvec, bp, d_vec, op); break;
+        case 2: e = launch_reduce1<SRC, 2>(mode, bias_first != 0, s, tab, W, nvec, bp, d_vec, op); break;
+        case 4: e = launch_reduce1<SRC, 4>(mode, bias_first != 0, s, tab, W, nvec, bp, d_vec, op); break;
+        case 8: e = launch_reduce1<SRC, 8>(mode, bias_first != 0, s, tab, W, nvec, bp, d_vec, op); break;
+        default: e = launch_reduce1<SRC, 0>(mode, bias_first != 0, s, tab, W, nvec, bp, d_vec, op); break;
     }
     return (int)e;
+}
+
+extern "C" int kr_reduce_bf16(const void* stack, int W, int64_t slice_stride, int64_t numel, const void* bias,
+                              int64_t bias_numel, int64_t D, int bias_first, void* out, void* stream) {
+    int rc = check_reduce_common(stack, W, numel, out);
+    if (rc != KR_OK) return rc;
+    if (numel > 0 && (rc = check_stack(stack, slice_stride)) != KR_OK) return rc;
+    const int mode = reduce_bias_mode(bias, bias_numel, numel, D);
+    if (mode < 0) return mode;
+    if (numel == 0) return KR_OK;
+    const StackedPeers src{(const u32x4*)stack, slice_stride / 8};
+    return launch_reduce(src, W, numel, bias, mode, D, bias_first, out, stream);
+}
+
+extern "C" int kr_reduce_ptrs_bf16(const void* const* bufs, int W, int64_t numel, const void* bias,
+                                   int64_t bias_numel, int64_t D, int bias_first, void* out, void* stream) {
+    int rc = check_reduce_common(bufs, W, numel, out);
+    if (rc != KR_OK) return rc;
+    const int mode = reduce_bias_mode(bias, bias_numel, numel, D);
+    if (mode < 0) return mode;
+    if (numel == 0) return KR_OK;
+    PeerTab tab;
+    if ((rc = peer_tab_from_ptrs(tab, bufs, W)) != KR_OK) return rc;
+    return launch_reduce(tab, W, numel, bias, mode, D, bias_first, out, stream);
 }
 
 extern "C" int64_t kr_striped_share_numel(int64_t numel, int W, int64_t stripe_block, int rank) {
@@ -243,22 +280,41 @@ extern "C" int64_t kr_striped_share_numel(int64_t numel, int W, int64_t stripe_b
     return full * stripe_block + tail;
 }
 
+template <class SRC>
+static int launch_striped(const SRC& tab, int W, int64_t share, const void* bias, int64_t stripe_block,
+                          int rank, void* out, void* stream) {
+    if (bias != nullptr && !aligned16(bias)) return KR_ERR_ALIGNMENT;
+    const int64_t nvec = share / 8;
+    const int64_t blocks = (nvec + kThreads - 1) / kThreads;
+    if (blocks > 0x7fffffffLL || stripe_block / 8 > 0xffffffffLL) return KR_ERR_BAD_DIM;
+    hipLaunchKernelGGL(reduce_striped_kernel<SRC>, dim3((unsigned)blocks), dim3(kThreads), 0, (hipStream_t)stream, tab,
+                       W, nvec, (const u32x4*)bias, (uint32_t)(stripe_block / 8), rank, (u32x4*)out);
+    return (int)hipGetLastError();
+}
+
 extern "C" int kr_reduce_striped_bf16(const void* stack, int W, int64_t slice_stride, int64_t numel,
                                       const void* bias, int64_t stripe_block, int rank, void* out,
                                       void* stream) {
     const int64_t share = kr_striped_share_numel(numel, W, stripe_block, rank);
     if (share < 0) return (int)share;
     if (share == 0) return KR_OK;
-    int rc = check_reduce_common(stack, W, slice_stride, numel, out);
+    int rc = check_reduce_common(stack, W, numel, out);
     if (rc != KR_OK) return rc;
-    if (bias != nullptr && !aligned16(bias)) return KR_ERR_ALIGNMENT;
-    const int64_t nvec = share / 8;
-    const int64_t blocks = (nvec + kThreads - 1) / kThreads;
-    if (blocks > 0x7fffffffLL || stripe_block / 8 > 0xffffffffLL) return KR_ERR_BAD_DIM;
-    hipLaunchKernelGGL(reduce_striped_kernel, dim3((unsigned)blocks), dim3(kThreads), 0, (hipStream_t)stream,
-                       (const u32x4*)stack, W, slice_stride / 8, nvec, (const u32x4*)bias,
-                       (uint32_t)(stripe_block / 8), rank, (u32x4*)out);
-    return (int)hipGetLastError();
+    if ((rc = check_stack(stack, slice_stride)) != KR_OK) return rc;
+    const StackedPeers src{(const u32x4*)stack, slice_stride / 8};
+    return launch_striped(src, W, share, bias, stripe_block, rank, out, stream);
+}
+
+extern "C" int kr_reduce_striped_ptrs_bf16(const void* const* bufs, int W, int64_t numel, const void* bias,
+                                           int64_t stripe_block, int rank, void* out, void* stream) {
+    const int64_t share = kr_striped_share_numel(numel, W, stripe_block, rank);
+    if (share < 0) return (int)share;
+    if (share == 0) return KR_OK;
+    int rc = check_reduce_common(bufs, W, numel, out);
+    if (rc != KR_OK) return rc;
+    PeerTab tab;
+    if ((rc = peer_tab_from_ptrs(tab, bufs, W)) != KR_OK) return rc;
+    return launch_striped(tab, W, share, bias, stripe_block, rank, out, stream);
 }
 
 extern "C" int kr_reduce_rotated_bf16(const void* in, int W, int64_t rows, int64_t N, int rank, int acc_bf16,

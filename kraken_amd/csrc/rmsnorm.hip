@@ -1,4 +1,5 @@
-// Row kernels: W-way reduce + bias + RMSNorm in one pass, and stand-alone RMSNorm.
+// Row kernels: W-way reduce + bias + RMSNorm in one pass, and stand-alone RMSNorm.  The W
+// inputs are the slices of a stacked tensor or the entries of a pointer table (SRC, common.h).
 //
 // One workgroup owns one row.  The reduced row lives in fp32 registers (VPT
 // 128-bit vectors per thread), so every input byte is read exactly once:
@@ -17,9 +18,9 @@ enum RowBias { kRowNoBias = 0, kRowFullBias = 1, kRowVecBias = 2 };
 constexpr int kMaxVpt = 8;       // vectors per thread  -> D <= 1024 * 8 * 8
 constexpr int kMaxThreads = 1024;
 
-template <int VPT, int WT, int BIAS>
+template <class SRC, int VPT, int WT, int BIAS>
 __global__ __launch_bounds__(kMaxThreads) void reduce_rmsnorm_kernel(
-    const u32x4* __restrict__ stack, int w_rt, int64_t slice_stride_v, int d_vec,
+    const SRC src, int w_rt, int d_vec,
     const u32x4* __restrict__ bias, const u32x4* __restrict__ wgt, float eps, float inv_d,
     u32x4* __restrict__ y) {
     __shared__ float wave_part[kMaxThreads / kWave];
@@ -63,7 +64,7 @@ __global__ __launch_bounds__(kMaxThreads) void reduce_rmsnorm_kernel(
 #pragma unroll
             for (int v = 0; v < VPT; ++v) {
                 const int c = tid + v * nthr;
-                x[r][v] = c < d_vec ? ld_stream(stack + r * slice_stride_v + row_v + c) : u32x4{0, 0, 0, 0};
+                x[r][v] = c < d_vec ? ld_stream(src.at(r) + row_v + c) : u32x4{0, 0, 0, 0};
             }
 #pragma unroll
         for (int r = 0; r < WT; ++r)
@@ -81,7 +82,7 @@ __global__ __launch_bounds__(kMaxThreads) void reduce_rmsnorm_kernel(
                 for (int v = 0; v < VPT; ++v) {
                     const int c = tid + v * nthr;
                     x[gi][v] = (r0 + gi < W && c < d_vec)
-                                   ? ld_stream(stack + (r0 + gi) * slice_stride_v + row_v + c)
+                                   ? ld_stream(src.at(r0 + gi) + row_v + c)
                                    : u32x4{0, 0, 0, 0};
                 }
 #pragma unroll
@@ -121,37 +122,37 @@ __global__ __launch_bounds__(kMaxThreads) void reduce_rmsnorm_kernel(
     }
 }
 
-template <int VPT, int WT>
-static hipError_t launch_row2(int mode, dim3 grid, dim3 block, hipStream_t st, const u32x4* stack, int W,
-                              int64_t ssv, int d_vec, const u32x4* bias, const u32x4* wgt, float eps,
+template <class SRC, int VPT, int WT>
+static hipError_t launch_row2(int mode, dim3 grid, dim3 block, hipStream_t st, const SRC& tab, int W,
+                              int d_vec, const u32x4* bias, const u32x4* wgt, float eps,
                               float inv_d, u32x4* y) {
     switch (mode) {
         case kRowNoBias:
-            hipLaunchKernelGGL((reduce_rmsnorm_kernel<VPT, WT, kRowNoBias>), grid, block, 0, st, stack, W, ssv,
+            hipLaunchKernelGGL((reduce_rmsnorm_kernel<SRC, VPT, WT, kRowNoBias>), grid, block, 0, st, tab, W,
                                d_vec, bias, wgt, eps, inv_d, y);
             break;
         case kRowFullBias:
-            hipLaunchKernelGGL((reduce_rmsnorm_kernel<VPT, WT, kRowFullBias>), grid, block, 0, st, stack, W, ssv,
+            hipLaunchKernelGGL((reduce_rmsnorm_kernel<SRC, VPT, WT, kRowFullBias>), grid, block, 0, st, tab, W,
                                d_vec, bias, wgt, eps, inv_d, y);
             break;
         default:
-            hipLaunchKernelGGL((reduce_rmsnorm_kernel<VPT, WT, kRowVecBias>), grid, block, 0, st, stack, W, ssv,
+            hipLaunchKernelGGL((reduce_rmsnorm_kernel<SRC, VPT, WT, kRowVecBias>), grid, block, 0, st, tab, W,
                                d_vec, bias, wgt, eps, inv_d, y);
             break;
     }
     return hipGetLastError();
 }
 
-template <int VPT>
-static hipError_t launch_row1(int W, int mode, dim3 grid, dim3 block, hipStream_t st, const u32x4* stack,
-                              int64_t ssv, int d_vec, const u32x4* bias, const u32x4* wgt, float eps,
+template <class SRC, int VPT>
+static hipError_t launch_row1(int W, int mode, dim3 grid, dim3 block, hipStream_t st, const SRC& tab,
+                              int d_vec, const u32x4* bias, const u32x4* wgt, float eps,
                               float inv_d, u32x4* y) {
     switch (W) {
-        case 1: return launch_row2<VPT, 1>(mode, grid, block, st, stack, W, ssv, d_vec, bias, wgt, eps, inv_d, y);
-        case 2: return launch_row2<VPT, 2>(mode, grid, block, st, stack, W, ssv, d_vec, bias, wgt, eps, inv_d, y);
-        case 4: return launch_row2<VPT, 4>(mode, grid, block, st, stack, W, ssv, d_vec, bias, wgt, eps, inv_d, y);
-        case 8: return launch_row2<VPT, 8>(mode, grid, block, st, stack, W, ssv, d_vec, bias, wgt, eps, inv_d, y);
-        default: return launch_row2<VPT, 0>(mode, grid, block, st, stack, W, ssv, d_vec, bias, wgt, eps, inv_d, y);
+        case 1: return launch_row2<SRC, VPT, 1>(mode, grid, block, st, tab, W, d_vec, bias, wgt, eps, inv_d, y);
+        case 2: return launch_row2<SRC, VPT, 2>(mode, grid, block, st, tab, W, d_vec, bias, wgt, eps, inv_d, y);
+        case 4: return launch_row2<SRC, VPT, 4>(mode, grid, block, st, tab, W, d_vec, bias, wgt, eps, inv_d, y);
+        case 8: return launch_row2<SRC, VPT, 8>(mode, grid, block, st, tab, W, d_vec, bias, wgt, eps, inv_d, y);
+        default: return launch_row2<SRC, VPT, 0>(mode, grid, block, st, tab, W, d_vec, bias, wgt, eps, inv_d, y);
     }
 }
 
@@ -174,25 +175,24 @@ static void row_geometry(int d_vec, int* threads, int* vpt) {
     *vpt = v;
 }
 
-static int launch_rows(const void* stack, int W, int64_t slice_stride, int64_t rows, int64_t D, const void* bias,
+template <class SRC>
+static int launch_rows(const SRC& tab, int W, int64_t rows, int64_t D, const void* bias,
                        int mode, const void* w, float eps, void* y, void* stream) {
     int threads, vpt;
     const int d_vec = (int)(D / 8);
     row_geometry(d_vec, &threads, &vpt);
     const dim3 grid((unsigned)rows), block((unsigned)threads);
     const hipStream_t st = (hipStream_t)stream;
-    const u32x4* sp = (const u32x4*)stack;
     const u32x4* bp = (const u32x4*)bias;
     const u32x4* wp = (const u32x4*)w;
     u32x4* yp = (u32x4*)y;
-    const int64_t ssv = slice_stride / 8;
     const float inv_d = 1.0f / (float)D;
     hipError_t e;
     switch (vpt) {
-        case 1: e = launch_row1<1>(W, mode, grid, block, st, sp, ssv, d_vec, bp, wp, eps, inv_d, yp); break;
-        case 2: e = launch_row1<2>(W, mode, grid, block, st, sp, ssv, d_vec, bp, wp, eps, inv_d, yp); break;
-        case 4: e = launch_row1<4>(W, mode, grid, block, st, sp, ssv, d_vec, bp, wp, eps, inv_d, yp); break;
-        default: e = launch_row1<8>(W, mode, grid, block, st, sp, ssv, d_vec, bp, wp, eps, inv_d, yp); break;
+        case 1: e = launch_row1<SRC, 1>(W, mode, grid, block, st, tab, d_vec, bp, wp, eps, inv_d, yp); break;
+        case 2: e = launch_row1<SRC, 2>(W, mode, grid, block, st, tab, d_vec, bp, wp, eps, inv_d, yp); break;
+        case 4: e = launch_row1<SRC, 4>(W, mode, grid, block, st, tab, d_vec, bp, wp, eps, inv_d, yp); break;
+        default: e = launch_row1<SRC, 8>(W, mode, grid, block, st, tab, d_vec, bp, wp, eps, inv_d, yp); break;
     }
     return (int)e;
 }
@@ -201,30 +201,51 @@ static int launch_rows(const void* stack, int W, int64_t slice_stride, int64_t r
 
 using namespace kr;
 
-extern "C" int kr_reduce_rmsnorm_bf16(const void* stack, int W, int64_t slice_stride, int64_t rows, int64_t D,
-                                      const void* bias, int bias_is_vector, const void* w, float eps, void* y,
-                                      void* stream) {
+// Argument checks shared by the row entry points (everything but the input buffers).
+// Returns KR_OK also for rows == 0.
+static int check_rows(int W, int64_t rows, int64_t D, const void* bias, const void* w, const void* y) {
     if (W < 1 || W > KR_MAX_WORLD) return KR_ERR_WORLD_SIZE;
-    if (rows < 0 || D <= 0 || slice_stride < 0) return KR_ERR_BAD_DIM;
-    if (D % 8 != 0) return KR_ERR_NUMEL_MOD8;
-    if (D > KR_MAX_ROW) return KR_ERR_ROW_TOO_LONG;
-    if (rows > 0x7fffffffLL) return KR_ERR_BAD_DIM;
-    if (rows == 0) return KR_OK;
-    if (stack == nullptr || w == nullptr || y == nullptr) return KR_ERR_NULL_POINTER;
-    if (!aligned16(stack) || !aligned16(w) || !aligned16(y) || slice_stride % 8 != 0) return KR_ERR_ALIGNMENT;
-    if (bias != nullptr && !aligned16(bias)) return KR_ERR_ALIGNMENT;
-    const int mode = bias == nullptr ? kRowNoBias : (bias_is_vector ? kRowVecBias : kRowFullBias);
-    return launch_rows(stack, W, slice_stride, rows, D, bias, mode, w, eps, y, stream);
-}
-
-extern "C" int kr_rmsnorm_bf16(const void* x, const void* w, float eps, int64_t rows, int64_t D, void* y,
-                               void* stream) {
     if (rows < 0 || D <= 0) return KR_ERR_BAD_DIM;
     if (D % 8 != 0) return KR_ERR_NUMEL_MOD8;
     if (D > KR_MAX_ROW) return KR_ERR_ROW_TOO_LONG;
     if (rows > 0x7fffffffLL) return KR_ERR_BAD_DIM;
     if (rows == 0) return KR_OK;
-    if (x == nullptr || w == nullptr || y == nullptr) return KR_ERR_NULL_POINTER;
-    if (!aligned16(x) || !aligned16(w) || !aligned16(y)) return KR_ERR_ALIGNMENT;
-    return launch_rows(x, 1, 0, rows, D, nullptr, kRowNoBias, w, eps, y, stream);
+    if (w == nullptr || y == nullptr) return KR_ERR_NULL_POINTER;
+    if (!aligned16(w) || !aligned16(y)) return KR_ERR_ALIGNMENT;
+    if (bias != nullptr && !aligned16(bias)) return KR_ERR_ALIGNMENT;
+    return KR_OK;
+}
+
+extern "C" int kr_reduce_rmsnorm_bf16(const void* stack, int W, int64_t slice_stride, int64_t rows, int64_t D,
+                                      const void* bias, int bias_is_vector, const void* w, float eps, void* y,
+                                      void* stream) {
+    if (W >= 1 && W <= KR_MAX_WORLD && slice_stride < 0) return KR_ERR_BAD_DIM;
+    int rc = check_rows(W, rows, D, bias, w, y);
+    if (rc != KR_OK || rows == 0) return rc;
+    if (stack == nullptr) return KR_ERR_NULL_POINTER;
+    if (!aligned16(stack) || slice_stride % 8 != 0) return KR_ERR_ALIGNMENT;
+    const int mode = bias == nullptr ? kRowNoBias : (bias_is_vector ? kRowVecBias : kRowFullBias);
+    const StackedPeers src{(const u32x4*)stack, slice_stride / 8};
+    return launch_rows(src, W, rows, D, bias, mode, w, eps, y, stream);
+}
+
+extern "C" int kr_reduce_rmsnorm_ptrs_bf16(const void* const* bufs, int W, int64_t rows, int64_t D,
+                                           const void* bias, int bias_is_vector, const void* w, float eps,
+                                           void* y, void* stream) {
+    int rc = check_rows(W, rows, D, bias, w, y);
+    if (rc != KR_OK || rows == 0) return rc;
+    PeerTab tab;
+    if ((rc = peer_tab_from_ptrs(tab, bufs, W)) != KR_OK) return rc;
+    const int mode = bias == nullptr ? kRowNoBias : (bias_is_vector ? kRowVecBias : kRowFullBias);
+    return launch_rows(tab, W, rows, D, bias, mode, w, eps, y, stream);
+}
+
+extern "C" int kr_rmsnorm_bf16(const void* x, const void* w, float eps, int64_t rows, int64_t D, void* y,
+                               void* stream) {
+    int rc = check_rows(1, rows, D, nullptr, w, y);
+    if (rc != KR_OK || rows == 0) return rc;
+    if (x == nullptr) return KR_ERR_NULL_POINTER;
+    if (!aligned16(x)) return KR_ERR_ALIGNMENT;
+    const StackedPeers src{(const u32x4*)x, 0};
+    return launch_rows(src, 1, rows, D, nullptr, kRowNoBias, w, eps, y, stream);
 }

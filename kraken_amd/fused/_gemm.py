@@ -1,6 +1,8 @@
 """Shared host logic of the GEMM + reduce wrappers."""
 from __future__ import annotations
 
+import ctypes
+
 import torch
 
 from .. import _lib
@@ -48,20 +50,47 @@ def prepare_operands(a: torch.Tensor, b: torch.Tensor) -> tuple[torch.Tensor, to
 
 
 def launch(name, a, b, M, N, peers, n_peers, peers_stride, bias, band_row0, band_rows, c_full, out, pivot):
-    dev = _lib.require_device(a, b, peers, bias, c_full, out)
-    rc = _lib.load().kr_gemm_reduce_bf16(
-        a.data_ptr(), a.stride(0), a.stride(1), b.data_ptr(), b.stride(0), b.stride(1),
-        M, N, a.shape[1], _lib.ptr(peers), n_peers, peers_stride, _lib.ptr(bias),
-        band_row0, band_rows, _lib.ptr(c_full), _lib.ptr(out),
-        int(out is not None and out.dtype == torch.float32), pivot, _lib.current_stream(dev),
-    )
+    """One call of the GEMM entry point; ``peers`` is a ``[P, rows, N]`` tensor (stacked entry
+    point), a list of P tensors (pointer-table entry point) or ``None``."""
+    lib = _lib.load()
+    out_fp32 = int(out is not None and out.dtype == torch.float32)
+    if isinstance(peers, (list, tuple)):
+        dev = _lib.require_device(a, b, *peers, bias, c_full, out)
+        table = (ctypes.c_void_p * max(n_peers, 1))(*[t.data_ptr() for t in peers])
+        rc = lib.kr_gemm_reduce_ptrs_bf16(
+            a.data_ptr(), a.stride(0), a.stride(1), b.data_ptr(), b.stride(0), b.stride(1),
+            M, N, a.shape[1], table, n_peers, _lib.ptr(bias),
+            band_row0, band_rows, _lib.ptr(c_full), _lib.ptr(out), out_fp32, pivot, _lib.current_stream(dev),
+        )
+    else:
+        dev = _lib.require_device(a, b, peers, bias, c_full, out)
+        rc = lib.kr_gemm_reduce_bf16(
+            a.data_ptr(), a.stride(0), a.stride(1), b.data_ptr(), b.stride(0), b.stride(1),
+            M, N, a.shape[1], _lib.ptr(peers), n_peers, peers_stride, _lib.ptr(bias),
+            band_row0, band_rows, _lib.ptr(c_full), _lib.ptr(out), out_fp32, pivot, _lib.current_stream(dev),
+        )
     _lib.check(rc, name)
 
 
-def check_peers(peers: torch.Tensor | None, rows: int, N: int) -> tuple[int, int]:
-    """Validate pre-staged partials ``[P, rows, N]``; return (P, stride)."""
+def n_peers_of(peers) -> int:
+    """Number of pre-staged partials in a ``peers`` argument (tensor, sequence or ``None``)."""
+    if peers is None:
+        return 0
+    return len(peers) if isinstance(peers, (list, tuple)) else peers.shape[0]
+
+
+def check_peers(peers, rows: int, N: int) -> tuple[int, int]:
+    """Validate pre-staged partials — one ``[P, rows, N]`` tensor or a sequence of P
+    ``[rows, N]`` tensors (separate allocations); return (P, stride), stride 0 for a sequence."""
     if peers is None:
         return 0, 0
+    if isinstance(peers, (list, tuple)):
+        for t in peers:
+            assert t.dtype == torch.bfloat16, "pre-staged partials must be bfloat16"
+            assert tuple(t.shape) == (rows, N) and t.is_contiguous(), (
+                f"every peer must be a contiguous [{rows}, {N}] tensor, got {tuple(t.shape)}"
+            )
+        return len(peers), 0
     assert peers.dtype == torch.bfloat16, "pre-staged partials must be bfloat16"
     assert peers.dim() == 3 and tuple(peers.shape[1:]) == (rows, N), (
         f"peers must have shape [W-1, {rows}, {N}], got {tuple(peers.shape)}"

@@ -16,8 +16,8 @@ def gemm_one_shot_all_reduce(a: torch.Tensor, b: torch.Tensor, **kwargs) -> torc
     other ranks arrive pre-staged and this rank's partial never leaves the
     accumulators.  kwargs:
 
-    * ``peers``: bf16 ``[W-1, M, N]`` partial products of the other ranks, or
-      ``None`` (W = 1: plain GEMM);
+    * ``peers``: bf16 ``[W-1, M, N]`` partial products of the other ranks (or a
+      list of W-1 separate ``[M, N]`` tensors), or ``None`` (W = 1: plain GEMM);
     * ``bias``: bf16 ``[N]`` or ``None`` (the reference has no bias here);
     * ``out_dtype``: ``torch.float32`` (default — the reference's output
       dtype, ``:135``) or ``torch.bfloat16``.

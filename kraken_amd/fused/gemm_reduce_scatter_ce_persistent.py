@@ -53,7 +53,7 @@ def gemm_reduce_scatter_ce_persistent(
     a2, b2 = _gemm.prepare_operands(a, b)
     M, N = a2.shape[0], b2.shape[1]
     peers = kwargs.get("peers")
-    world_size = kwargs.get("world_size", (peers.shape[0] + 1) if peers is not None else 1)
+    world_size = kwargs.get("world_size", _gemm.n_peers_of(peers) + 1)
     rank = kwargs.get("rank", 0)
     assert M % world_size == 0
     m_per_rank = M // world_size

@@ -19,8 +19,8 @@ def gemm_reduce_scatter(a: torch.Tensor, b: torch.Tensor, **kwargs) -> torch.Ten
     stays in fp32 (the reference rounds it to the input dtype first, ``:72``).
     kwargs:
 
-    * ``peers``: bf16 ``[W-1, M/W, N]`` — the other ranks' partials of this
-      rank's band; ``None`` means W = ``world_size`` (default 1) without peers;
+    * ``peers``: bf16 ``[W-1, M/W, N]`` (or a list of W-1 separate ``[M/W, N]``
+      tensors) — the other ranks' partials of this rank's band; ``None`` means W = ``world_size`` (default 1) without peers;
     * ``rank`` (default 0), ``world_size`` (default ``len(peers)+1``);
     * ``c_scratch``: bf16 ``[M, N]`` buffer for the other bands; allocated if
       ``None``; pass ``False`` to skip writing them.
@@ -32,7 +32,7 @@ def gemm_reduce_scatter(a: torch.Tensor, b: torch.Tensor, **kwargs) -> torch.Ten
     M, N = a.shape[0], b.shape[1]
     assert N % 8 == 0, "N must be a multiple of 8"
     peers = kwargs.get("peers")
-    world_size = kwargs.get("world_size", (peers.shape[0] + 1) if peers is not None else 1)
+    world_size = kwargs.get("world_size", _gemm.n_peers_of(peers) + 1)
     rank = kwargs.get("rank", 0)
     assert M % world_size == 0, f"M dimension ({M}) must be divisible by world_size ({world_size})"
     assert 0 <= rank < world_size

@@ -8,7 +8,7 @@ from ..comm._common import bias_args, check_stack, stage_input
 
 
 def one_shot_all_reduce_bias(
-    symm_mem_buffer: torch.Tensor,
+    symm_mem_buffer,
     input_tensor: torch.Tensor | None,
     bias: torch.Tensor | None,
     output: torch.Tensor,
@@ -24,7 +24,7 @@ def one_shot_all_reduce_bias(
     (``kraken/fused/one_shot_all_reduce_bias.py:105-173``; arithmetic ``:76-94``).
 
     ``symm_mem_buffer`` is the ``[W, ...]`` stack standing in for the peers'
-    symmetric-memory buffers; each slice may be larger than the input, only its
+    symmetric-memory buffers, or a list of W separate tensors; each slice may be larger than the input, only its
     first ``output.numel()`` elements are used (the reference rendezvouses on a
     buffer larger than the message as well, ``test/test_allreduce_bias.py:57-62``).
     ``input_tensor``, if given, is first copied into slice ``rank`` — the
@@ -35,7 +35,8 @@ def one_shot_all_reduce_bias(
     """
     if symm_mem_buffer is None:
         raise ValueError("symm_mem_buffer much be a valid symmetric memory tensor.")
-    W, cap, stride = check_stack(symm_mem_buffer)
+    peers = check_stack(symm_mem_buffer)
+    W, cap = peers.W, peers.cap
     ref = input_tensor if input_tensor is not None else output
     assert ref.dtype == torch.bfloat16, "Only bfloat16 is supported for now."
     numel = ref.numel()
@@ -45,10 +46,7 @@ def one_shot_all_reduce_bias(
     assert 0 <= rank < W
     D = ref.shape[-1] if ref.dim() >= 1 else numel
     bias_ptr, bias_numel = bias_args(bias, numel, D)
-    dev = _lib.require_device(symm_mem_buffer, input_tensor, bias, output)
-    stage_input(symm_mem_buffer, input_tensor, rank)
-    rc = _lib.load().kr_reduce_bf16(
-        symm_mem_buffer.data_ptr(), W, stride, numel, bias_ptr, bias_numel, D, 1,
-        output.data_ptr(), _lib.current_stream(dev),
-    )
+    dev = _lib.require_device(*peers.tensors, input_tensor, bias, output)
+    stage_input(peers, input_tensor, rank)
+    rc = peers.reduce(0, numel, bias_ptr, bias_numel, D, 1, output.data_ptr(), _lib.current_stream(dev))
     _lib.check(rc, "one_shot_all_reduce_bias")

@@ -21,7 +21,8 @@ def _launch_reduce_rms_norm(name, symm_mem_input, x, bias, w, y, eps, rank):
     assert y.is_contiguous()
     assert y.dtype == torch.bfloat16 and w.dtype == torch.bfloat16, "Only bfloat16 is supported for now."
     assert D % 8 == 0, "The row length must be 128-bit aligned."
-    W, cap, stride = check_stack(symm_mem_input)
+    peers = check_stack(symm_mem_input)
+    W, cap = peers.W, peers.cap
     rows = math.prod(y.shape[:-1])
     assert rows * D <= cap, "the message does not fit in one slice of the stacked buffer"
     assert 0 <= rank < W
@@ -30,17 +31,15 @@ def _launch_reduce_rms_norm(name, symm_mem_input, x, bias, w, y, eps, rank):
         assert bias.dtype == torch.bfloat16 and bias.is_contiguous()
         assert bias.numel() in (rows * D, D), "bias must have the shape of x or be a vector of the last dim"
         bias_is_vector = int(bias.numel() == D and rows != 1)
-    dev = _lib.require_device(symm_mem_input, x, bias, w, y)
-    stage_input(symm_mem_input, x, rank)
-    rc = _lib.load().kr_reduce_rmsnorm_bf16(
-        symm_mem_input.data_ptr(), W, stride, rows, D, _lib.ptr(bias), bias_is_vector, w.data_ptr(),
-        float(eps), y.data_ptr(), _lib.current_stream(dev),
-    )
+    dev = _lib.require_device(*peers.tensors, x, bias, w, y)
+    stage_input(peers, x, rank)
+    rc = peers.reduce_rmsnorm(rows, D, _lib.ptr(bias), bias_is_vector, w.data_ptr(), float(eps), y.data_ptr(),
+                              _lib.current_stream(dev))
     _lib.check(rc, name)
 
 
 def one_shot_all_reduce_bias_rms_norm(
-    symm_mem_input: torch.Tensor,
+    symm_mem_input,
     x: torch.Tensor | None,
     bias: torch.Tensor | None,
     w: torch.Tensor,
@@ -58,7 +57,8 @@ def one_shot_all_reduce_bias_rms_norm(
     ``:73-91``): per row, ``s = fp32(bias) + x_0 + ... + x_{W-1}`` in fp32,
     ``y = bf16(s * rsqrt(mean(s^2) + eps) * fp32(w))``.
 
-    ``symm_mem_input`` is the ``[W, ...]`` stack; ``x``, if given, is copied
+    ``symm_mem_input`` is the ``[W, ...]`` stack or a list of W separate
+    tensors; ``x``, if given, is copied
     into slice ``rank`` first (the reference's copy-in ``:57-61``), pass
     ``None`` when the stack is already staged.  ``bias`` has the shape of
     ``x`` (reference usage) or ``[D]``.  ``BLOCK_SIZE``/``group`` are ignored.

@@ -8,7 +8,7 @@ from ..comm._common import bias_args, check_stack, stage_input
 
 
 def two_shot_all_reduce_bias(
-    symm_mem_input: torch.Tensor,
+    symm_mem_input,
     input_tensor: torch.Tensor | None,
     bias: torch.Tensor | None,
     output: torch.Tensor,
@@ -33,12 +33,14 @@ def two_shot_all_reduce_bias(
       ``layout="striped"`` — the reference's interleaved ownership with stripe
       block ``BLOCK_SIZE`` (``:66-69``), written compactly.
 
-    The message length is ``input_tensor.numel()`` if an input is given
+    ``symm_mem_input`` is the ``[W, ...]`` stack or a list of W separate
+    tensors.  The message length is ``input_tensor.numel()`` if an input is given
     (it is first copied into slice ``rank``, the reference's copy-in
     ``:43-50``), else ``numel`` if passed, else ``bias.numel()`` for a
     full-shape bias, else the slice size.  Returns ``output``.
     """
-    W, cap, stride = check_stack(symm_mem_input)
+    peers = check_stack(symm_mem_input)
+    W, cap = peers.W, peers.cap
     assert BLOCK_SIZE % W == 0
     assert layout in ("rows", "striped")
     assert 0 <= rank < W
@@ -54,20 +56,18 @@ def two_shot_all_reduce_bias(
     assert n % 8 == 0, "The number of elements must be 128-bit aligned."
     assert n <= cap, "the message does not fit in one slice of the stacked buffer"
     assert output.dtype == torch.bfloat16 and output.is_contiguous()
-    ref = input_tensor if input_tensor is not None else symm_mem_input[0]
+    ref = input_tensor if input_tensor is not None else peers.slice(0)
     D = ref.shape[-1]
     if bias is not None:
         assert bias.dtype == torch.bfloat16 and bias.is_contiguous()
-    dev = _lib.require_device(symm_mem_input, input_tensor, bias, output)
-    stage_input(symm_mem_input, input_tensor, rank)
+    dev = _lib.require_device(*peers.tensors, input_tensor, bias, output)
+    stage_input(peers, input_tensor, rank)
     lib = _lib.load()
     stream = _lib.current_stream(dev)
 
     if output.numel() == n:  # every share: the full result
         bias_ptr, bias_numel = bias_args(bias, n, D)
-        rc = lib.kr_reduce_bf16(
-            symm_mem_input.data_ptr(), W, stride, n, bias_ptr, bias_numel, D, 0, output.data_ptr(), stream
-        )
+        rc = peers.reduce(0, n, bias_ptr, bias_numel, D, 0, output.data_ptr(), stream)
         _lib.check(rc, "two_shot_all_reduce_bias")
         return output
 
@@ -77,9 +77,7 @@ def two_shot_all_reduce_bias(
         assert output.numel() == share, f"output must hold the {share} elements rank {rank} owns"
         if bias is not None:
             assert bias.numel() == n, "striped ownership needs a bias of the input's shape"
-        rc = lib.kr_reduce_striped_bf16(
-            symm_mem_input.data_ptr(), W, stride, n, _lib.ptr(bias), BLOCK_SIZE, rank, output.data_ptr(), stream
-        )
+        rc = peers.reduce_striped(n, _lib.ptr(bias), BLOCK_SIZE, rank, output.data_ptr(), stream)
         _lib.check(rc, "two_shot_all_reduce_bias")
         return output
 
@@ -95,9 +93,6 @@ def two_shot_all_reduce_bias(
         else:
             assert bias.numel() == D and share % D == 0, "a vector bias needs shares made of whole rows"
             bias_ptr, bias_numel = bias.data_ptr(), D
-    rc = lib.kr_reduce_bf16(
-        symm_mem_input.data_ptr() + 2 * off, W, stride, share, bias_ptr, bias_numel, D, 0,
-        output.data_ptr(), stream,
-    )
+    rc = peers.reduce(off, share, bias_ptr, bias_numel, D, 0, output.data_ptr(), stream)
     _lib.check(rc, "two_shot_all_reduce_bias")
     return output

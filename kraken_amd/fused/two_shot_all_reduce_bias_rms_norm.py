@@ -10,7 +10,7 @@ from .one_shot_all_reduce_bias_rms_norm import _launch_reduce_rms_norm
 
 
 def two_shot_all_reduce_bias_rms_norm(
-    symm_mem_input: torch.Tensor,
+    symm_mem_input,
     x: torch.Tensor | None,
     bias: torch.Tensor | None,
     w: torch.Tensor,
@@ -42,7 +42,7 @@ def two_shot_all_reduce_bias_rms_norm(
         rows_per_block = 4
     else:
         rows_per_block = 8
-    W, _, _ = check_stack(symm_mem_input)
+    W = check_stack(symm_mem_input).W
     size_per_rank = rows_per_block * D // W
     assert size_per_rank * W == rows_per_block * D
     assert size_per_rank % 16 == 0

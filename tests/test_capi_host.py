@@ -91,6 +91,74 @@ def test_gemm_argument_errors(lib):
     assert call(M=0, band=0) == 0
 
 
+def _table(*ptrs):
+    return (ctypes.c_void_p * len(ptrs))(*ptrs)
+
+
+def test_pointer_table_argument_errors(lib):
+    """The kr_*_ptrs_bf16 forms reject what their stacked forms reject, and a bad table entry."""
+    good = _table(*[FAKE + 4096 * r for r in range(8)])
+    f = lib.kr_reduce_ptrs_bf16
+    assert f(good, 8, 12, None, 0, 0, 1, FAKE, None) == _lib.KR_ERR_NUMEL_MOD8
+    assert f(good, 0, 16, None, 0, 0, 1, FAKE, None) == _lib.KR_ERR_WORLD_SIZE
+    assert f(good, 17, 16, None, 0, 0, 1, FAKE, None) == _lib.KR_ERR_WORLD_SIZE
+    assert f(None, 8, 16, None, 0, 0, 1, FAKE, None) == _lib.KR_ERR_NULL_POINTER
+    assert f(good, 8, 16, None, 0, 0, 1, None, None) == _lib.KR_ERR_NULL_POINTER
+    assert f(_table(FAKE, None), 2, 16, None, 0, 0, 1, FAKE, None) == _lib.KR_ERR_NULL_POINTER
+    assert f(_table(FAKE, FAKE + 8), 2, 16, None, 0, 0, 1, FAKE, None) == _lib.KR_ERR_ALIGNMENT
+    assert f(good, 8, 64, FAKE, 24, 16, 1, FAKE, None) == _lib.KR_ERR_BIAS_SHAPE
+    assert f(good, 8, -8, None, 0, 0, 1, FAKE, None) == _lib.KR_ERR_BAD_DIM
+    assert f(None, 8, 0, None, 0, 0, 1, None, None) == 0
+
+    f = lib.kr_reduce_striped_ptrs_bf16
+    assert f(good, 8, 4096, None, 12, 0, FAKE, None) == _lib.KR_ERR_STRIPE
+    assert f(good, 8, 4096, None, 256, 8, FAKE, None) == _lib.KR_ERR_STRIPE
+    assert f(_table(FAKE, FAKE + 2), 2, 4096, None, 256, 0, FAKE, None) == _lib.KR_ERR_ALIGNMENT
+    assert f(None, 8, 4096, None, 256, 0, FAKE, None) == _lib.KR_ERR_NULL_POINTER
+    assert f(good, 8, 256, None, 256, 3, FAKE, None) == 0   # rank 3 owns nothing of a 256-element input
+
+    f = lib.kr_reduce_rmsnorm_ptrs_bf16
+    assert f(good, 8, 1, 4100, None, 0, FAKE, 1e-5, FAKE, None) == _lib.KR_ERR_NUMEL_MOD8
+    assert f(good, 8, 1, 65536 + 8, None, 0, FAKE, 1e-5, FAKE, None) == _lib.KR_ERR_ROW_TOO_LONG
+    assert f(good, 8, 1, 4096, None, 0, None, 1e-5, FAKE, None) == _lib.KR_ERR_NULL_POINTER
+    assert f(None, 8, 1, 4096, None, 0, FAKE, 1e-5, FAKE, None) == _lib.KR_ERR_NULL_POINTER
+    assert f(_table(FAKE + 6), 1, 1, 4096, None, 0, FAKE, 1e-5, FAKE, None) == _lib.KR_ERR_ALIGNMENT
+    assert f(good, 8, 0, 4096, None, 0, None, 1e-5, None, None) == 0
+
+    f = lib.kr_gemm_reduce_ptrs_bf16
+    def args(**kw):
+        a = dict(A=FAKE, lda_m=64, lda_k=1, B=FAKE, ldb_k=64, ldb_n=1, M=64, N=64, K=64, peers=None, n_peers=0,
+                 bias=None, band_row0=0, band_rows=64, c_full=None, out=FAKE, out_is_fp32=0, tile_pivot=0,
+                 stream=None)
+        a.update(kw)
+        return tuple(a.values())
+    assert f(*args(n_peers=2, peers=None)) == _lib.KR_ERR_NULL_POINTER
+    assert f(*args(n_peers=2, peers=_table(FAKE, None))) == _lib.KR_ERR_NULL_POINTER
+    assert f(*args(n_peers=2, peers=_table(FAKE, FAKE + 4))) == _lib.KR_ERR_ALIGNMENT
+    assert f(*args(n_peers=16, peers=good)) == _lib.KR_ERR_WORLD_SIZE
+    assert f(*args(n_peers=2, peers=good, band_row0=32, band_rows=64)) == _lib.KR_ERR_BAND
+    assert f(*args(n_peers=2, peers=good, lda_k=2)) == _lib.KR_ERR_LAYOUT
+    assert f(*args(n_peers=2, peers=good, M=0, band_rows=0)) == 0
+
+
+def test_wrappers_accept_a_list_of_buffers_and_check_it():
+    bufs = [torch.zeros(4, 16, dtype=BF16) for _ in range(3)]
+    with pytest.raises(RuntimeError, match="no CPU fallback"):
+        comm.one_shot_all_reduce(bufs)
+    with pytest.raises(AssertionError, match="one shape"):
+        comm.one_shot_all_reduce([bufs[0], torch.zeros(4, 8, dtype=BF16)])
+    with pytest.raises(AssertionError, match="bfloat16"):
+        comm.one_shot_all_reduce([bufs[0], torch.zeros(4, 16)])
+    with pytest.raises(AssertionError, match="contiguous"):
+        comm.one_shot_all_reduce([bufs[0], torch.zeros(16, 4, dtype=BF16).T])
+    a = torch.zeros(8, 16, dtype=BF16)
+    b = torch.zeros(16, 8, dtype=BF16)
+    with pytest.raises(AssertionError, match="every peer"):
+        fused.gemm_one_shot_all_reduce_fused(a, b, peers=[torch.zeros(8, 16, dtype=BF16)])
+    with pytest.raises(RuntimeError, match="no CPU fallback"):
+        fused.gemm_one_shot_all_reduce_fused(a, b, peers=[torch.zeros(8, 8, dtype=BF16)])
+
+
 def test_striped_share_numel(lib):
     f = lib.kr_striped_share_numel
     numel, W, block = 8 * 37, 4, 16

@@ -253,6 +253,43 @@ def test_gemm_all_reduce_world_sizes(dev, tile, P):
         torch.testing.assert_close(outb.cpu(), want.to(BF16), **TOL)
 
 
+@pytest.mark.parametrize("P", [1, 3, 7, 15])
+def test_separate_peer_buffers_match_the_stacked_form(dev, tile, P):
+    """Pointer-table entry point: the peers' partial sums as P separate allocations give the
+    stacked form's bits, on whole-band 256-tiles (matrix-core path, 7-peer and generic epilogue
+    paths) and on a ragged shape."""
+    for (M, N, K) in [(512, 512, 192), (200, 136, 72)]:
+        a, b, peers = mk(M, N, K, P, seed=P)
+        bias = orc.randn_bf16((N,), 9, 0.02)
+        pads, plist = [], [None] * P
+        for j in reversed(range(P)):
+            pads.append(torch.empty(1208 * (j % 3 + 1), dtype=BF16, device=dev))
+            plist[j] = peers[j].to(dev)
+        ad, bd, pd, biasd = a.to(dev), b.to(dev), peers.to(dev), bias.to(dev)
+        for dt in (torch.float32, BF16):
+            o1 = fused.gemm_one_shot_all_reduce_fused(ad, bd, peers=pd, bias=biasd, out_dtype=dt)
+            o2 = fused.gemm_one_shot_all_reduce_fused(ad, bd, peers=plist, bias=biasd, out_dtype=dt)
+            assert torch.equal(o1, o2)
+        torch.testing.assert_close(o2.cpu(), orc.gemm_all_reduce(a, b, peers, bias).to(BF16), **TOL)
+    # reduce-scatter: band of rank 1 of W = P + 1, other bands to the scratch
+    W = P + 1
+    M, N, K = 256 * W, 256, 128
+    a, b, _ = mk(M, N, K, 0)
+    peers = torch.stack([orc.randn_bf16((M // W, N), 100 + j) for j in range(P)])
+    plist = [peers[j].to(dev) for j in range(P)]
+    c1 = torch.zeros(M, N, dtype=BF16, device=dev)
+    c2 = torch.zeros(M, N, dtype=BF16, device=dev)
+    o1 = fused.gemm_reduce_scatter(a.to(dev), b.to(dev), peers=peers.to(dev), rank=1, c_scratch=c1)
+    o2 = fused.gemm_reduce_scatter(a.to(dev), b.to(dev), peers=plist, rank=1, c_scratch=c2)
+    assert torch.equal(o1, o2) and torch.equal(c1, c2)
+    want, _ = orc.gemm_reduce_scatter(a, b, peers, 1, W)
+    torch.testing.assert_close(o2.cpu(), want, **TOL)
+    # the copy-engine variant takes a list as well
+    o3 = fused.gemm_reduce_scatter_ce_persistent(a.to(dev), b.to(dev), peers=plist, rank=1, world_size=W)
+    o4 = fused.gemm_reduce_scatter_ce_persistent(a.to(dev), b.to(dev), peers=peers.to(dev), rank=1, world_size=W)
+    assert torch.equal(o3, o4)
+
+
 def test_gemm_paths_replay_from_a_graph(dev, monkeypatch):
     """The GEMM entry point enqueues kernels only (no allocation, no memset, no host sync), so a
     caller may capture it: three fused calls are captured once and replayed with eager work in

@@ -94,6 +94,78 @@ def test_negative_zero_and_specials(dev):
     assert same_bits(out[ok], want[ok])
 
 
+def scattered(stack, dev):
+    """The W slices of a host stack as W separate device allocations, irregularly spaced and in
+    no address order (what a table of real peer mappings looks like)."""
+    W = stack.shape[0]
+    bufs, pads = [None] * W, []
+    for r in reversed(range(W)):
+        pads.append(torch.empty(1000 * (r % 3 + 1) + 8, dtype=BF16, device=dev))   # irregular gaps
+        bufs[r] = stack[r].to(dev)
+    return bufs
+
+
+@pytest.mark.parametrize("W", [1, 2, 3, 8, 16])
+def test_separate_buffers_match_the_stacked_form(dev, W):
+    """Pointer-table entry points: W separate allocations give the oracle's bits, i.e. the
+    same as the stacked form, for every reduce wrapper."""
+    rows, D = 45, 264
+    stack = orc.make_stack(W, (rows, D), seed0=11)
+    bufs = scattered(stack, dev)
+    assert same_bits(comm.one_shot_all_reduce(bufs), orc.reduce(stack))
+    assert same_bits(comm.two_shot_all_reduce(bufs, rank=None, BLOCK_SIZE=128 * W), orc.reduce(stack))
+    full_bias, vec_bias = orc.randn_bf16((rows, D), 7), orc.randn_bf16((D,), 8)
+    out = torch.empty(rows, D, dtype=BF16, device=dev)
+    for bias in (None, full_bias, vec_bias):
+        bd = None if bias is None else bias.to(dev)
+        fused.one_shot_all_reduce_bias(bufs, None, bd, out)
+        assert same_bits(out, orc.reduce(stack, bias, bias_first=True))
+        fused.two_shot_all_reduce_bias(bufs, None, bd, out, BLOCK_SIZE=128 * W)
+        assert same_bits(out, orc.reduce(stack, bias, bias_first=False))
+    # copy-in of this rank's input into its own buffer of the list
+    x = orc.randn_bf16((rows, D), 99)
+    rank = W - 1
+    fused.one_shot_all_reduce_bias(bufs, x.to(dev), full_bias.to(dev), out, rank=rank)
+    staged = stack.clone()
+    staged[rank] = x
+    assert same_bits(out, orc.reduce(staged, full_bias, bias_first=True))
+
+
+def test_separate_buffers_two_shot_shares(dev):
+    W, numel, block = 8, 2048 * 8 * 3 + 8 * 100, 2048
+    stack = orc.make_stack(W, (numel,), seed0=5)
+    bufs = scattered(stack, dev)
+    bias = orc.randn_bf16((numel,), 9)
+    full = orc.reduce(stack, bias, bias_first=False)
+    assembled = torch.empty_like(full)
+    for rank in range(W):
+        idx = orc.striped_indices(numel, W, block, rank)
+        share = comm.two_shot_all_reduce(bufs, rank=rank, layout="striped", BLOCK_SIZE=block)
+        assert same_bits(share, orc.reduce_striped(stack, None, block, rank))
+        out = torch.empty(idx.numel(), dtype=BF16, device=dev)
+        fused.two_shot_all_reduce_bias(bufs, None, bias.to(dev), out, BLOCK_SIZE=block, rank=rank,
+                                       layout="striped", numel=numel)
+        assembled[idx] = out.cpu()
+    assert same_bits(assembled, full)
+    # contiguous shares: every entry of the table is moved on by the share's offset
+    stack2 = orc.make_stack(W, (64, 256), seed0=6)
+    bufs2 = scattered(stack2, dev)
+    for rank in (0, 5, 7):
+        share = comm.two_shot_all_reduce(bufs2, rank=rank)
+        assert share.shape == (8, 256)
+        assert same_bits(share, orc.reduce(stack2[:, rank * 8:(rank + 1) * 8]))
+
+
+def test_separate_buffers_full_size_config2(dev):
+    """[8, 4096, 4096] as eight 32 MiB allocations: same bits as the stacked launch."""
+    W = 8
+    g = torch.Generator(device="cpu").manual_seed(3)
+    bufs = [torch.randn(4096, 4096, generator=g).to(BF16).to(dev) for _ in range(W)]
+    stack = torch.stack(bufs)
+    assert same_bits(comm.one_shot_all_reduce(bufs), comm.one_shot_all_reduce(stack))
+    del stack
+
+
 @pytest.mark.parametrize("rank", [0, 3, 7])
 def test_two_shot_row_share(dev, rank):
     W = 8

@@ -81,6 +81,34 @@ def test_world_sizes_and_bias_modes(dev, W, bias_mode):
     assert_one_ulp(y, want)
 
 
+@pytest.mark.parametrize("W,rows,D", [(1, 3, 64), (3, 9, 1000), (8, 16, 8192), (8, 5, 16384), (16, 2, 65536)])
+def test_separate_buffers_match_the_stacked_form(dev, W, rows, D):
+    """Pointer-table entry point: W separate allocations give exactly the stacked form's bits
+    (same kernel), for the short-row, grouped and long-row code paths."""
+    stack = orc.make_stack(W, (rows, D), seed0=21)
+    w = orc.randn_bf16((D,), 5, 0.02, 1.0)
+    pads, bufs = [], [None] * W
+    for r in reversed(range(W)):
+        pads.append(torch.empty(808 * (r % 3 + 1), dtype=BF16, device=dev))
+        bufs[r] = stack[r].to(dev)
+    sd = stack.to(dev)
+    for bias in (None, orc.randn_bf16((rows, D), 7), orc.randn_bf16((D,), 7, 0.02)):
+        bd = None if bias is None else bias.to(dev)
+        y1 = torch.empty(rows, D, dtype=BF16, device=dev)
+        y2 = torch.empty(rows, D, dtype=BF16, device=dev)
+        fused.one_shot_all_reduce_bias_rms_norm(sd, None, bd, w.to(dev), y1, eps=1e-5)
+        fused.one_shot_all_reduce_bias_rms_norm(bufs, None, bd, w.to(dev), y2, eps=1e-5)
+        assert torch.equal(y1.view(torch.int16), y2.view(torch.int16))
+        assert_one_ulp(y2, orc.reduce_bias_rms_norm(stack, bias, w, 1e-5))
+    if (rows * D) % (W * 16) == 0 and D % W == 0:
+        y3 = torch.empty(rows, D, dtype=BF16, device=dev)
+        x = orc.randn_bf16((rows, D), 31)
+        fused.two_shot_all_reduce_bias_rms_norm(bufs, x.to(dev), None, w.to(dev), y3, rank=0)
+        staged = stack.clone()
+        staged[0] = x
+        assert_one_ulp(y3, orc.reduce_bias_rms_norm(staged, None, w, 1e-5))
+
+
 def test_nd_input_and_eps(dev):
     W, B, T, D = 4, 3, 5, 512
     stack = orc.make_stack(W, (B, T, D))
