@@ -206,6 +206,47 @@ int kr_gemm_reduce_ptrs_bf16(const void* A, int64_t lda_m, int64_t lda_k,
                              int64_t tile_pivot, void* stream);
 
 /*
+ * All-gather matmul that consumes A while it is still arriving:  C[M,N] = A[M,K] @ B[K,N]  (bf16, fp32
+ * accumulate, bf16 result), where A is the gathered matrix of W shards of M/W rows, filled by
+ * copies that run on another stream while this kernel runs.  The rows arrive in W*splits_per_rank
+ * blocks of comm_rows = M / (W*splits_per_rank) rows; progress[b] is 0 until block b (rows
+ * [b*comm_rows, (b+1)*comm_rows)) is complete and is then set to 1 by kr_stream_write_value32
+ * behind the block's copy.  An output tile whose rows lie in the local shard (rows
+ * [rank*M/W, (rank+1)*M/W)) reads them from A_local [M/W, K] (row stride lda_local) and never
+ * waits; any other tile first waits until the flags of the blocks it covers are 1, then reads A.
+ * The order of the M tiles is rotated so that the local shard's tiles come first, the other
+ * shards following in the order rank+1, rank+2, ... in which the copies are issued.
+ *   A_local == NULL: local tiles wait for their flags and read A like the others.
+ *   progress == NULL: nothing waits (A is complete); A_local is then not used.
+ *   wait_limit_us: bound of one tile's wait in microseconds (<= 0: 5 s).  A tile whose flag does
+ *     not come in time stores 1 + block index to *status (if status != NULL; the caller zeroes
+ *     it beforehand), computes on whatever A holds and exits; tiles that start after that do
+ *     not wait.  The kernel therefore always ends; *status != 0 afterwards means C is invalid.
+ * A: k-contiguous, row stride lda_m; B as for kr_gemm_reduce_bf16; progress and status are
+ * device pointers, 4-byte aligned.  Requirements: M % (W*splits_per_rank) == 0, 0 <= rank < W,
+ * K % 8 == 0, N % 8 == 0.  The caller must have the copies (and their flag writes) enqueued
+ * on another stream before or right after this call, or the tiles wait until the limit.
+ *
+ * Replaces kraken/fused/all_gather_matmul.py:25-123 (_matmul_kernel_tma_persistent_w_progress;
+ * flag wait :95-110 = wait_gmem_barrier, kraken/_ptx_utils/gmem_barrier_arrive_wait.py:26-68)
+ * as launched by _matmul_w_progress (:147-219).
+ */
+int kr_all_gather_matmul_bf16(const void* A, int64_t lda_m, const void* A_local, int64_t lda_local,
+                              const void* B, int64_t ldb_k, int64_t ldb_n,
+                              int64_t M, int64_t N, int64_t K,
+                              int W, int rank, int splits_per_rank,
+                              const uint32_t* progress, int64_t wait_limit_us, int32_t* status,
+                              void* C, void* stream);
+
+/*
+ * Stream-ordered flag write: *addr = value once everything enqueued on `stream` before this call
+ * has completed, with its results visible to kernels that read the flag (release at system scope).
+ * Replaces symm_mem_hdl.stream_write_value32 as used behind every chunk copy of the
+ * copy-engine all-gather (kraken/comm/copy_engine_all_gather.py:47-53).
+ */
+int kr_stream_write_value32(uint32_t* addr, uint32_t value, void* stream);
+
+/*
  * Tile reduce of the copy-engine reduce-scatter variant: `in` is [W*rows, N]
  * bf16 (band r holds what rank r pushed), and
  *   out[m, n] = sum_{i=0..W-1} in[((i + rank + 1) % W) * rows + m, n]

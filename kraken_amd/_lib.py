@@ -61,6 +61,12 @@ _SIGNATURES = {
         [c_void_p, c_int64, c_int64, c_void_p, c_int64, c_int64, c_int64, c_int64, c_int64,
          c_void_p, c_int, c_int64, c_void_p, c_int64, c_int64, c_void_p, c_void_p, c_int, c_int64, c_void_p],
     ),
+    "kr_all_gather_matmul_bf16": (
+        c_int,
+        [c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_int64, c_int64, c_int64, c_int64, c_int64,
+         c_int, c_int, c_int, c_void_p, c_int64, c_void_p, c_void_p, c_void_p],
+    ),
+    "kr_stream_write_value32": (c_int, [c_void_p, ctypes.c_uint32, c_void_p]),
     "kr_reduce_rotated_bf16": (c_int, [c_void_p, c_int, c_int64, c_int64, c_int, c_int, c_void_p, c_void_p]),
 }
 

@@ -69,6 +69,9 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_reduce_kernel(const GemmArgs
     int tile_m, tile_n;
     tile_schedule(g, tile_m, tile_n);
     const int m0 = tile_m * BM, n0 = tile_n * BN;
+    const uint16_t* a_tile;   // first row of the tile's A panel (gathered matrix or local shard)
+    int64_t lda;
+    gathered_a_tile(g, m0, BM, a_tile, lda);
 
     f32x16 acc[TM][TN];
 #pragma unroll
@@ -98,7 +101,7 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_reduce_kernel(const GemmArgs
         const int row = (i * T + tid) >> 3;
         int m = m0 + row;
         if (!EVEN) m = min(m, g.M - 1);
-        a_goff[i] = (uint32_t)(((int64_t)(m - m0) * g.lda + ld_kc * 8) * 2);
+        a_goff[i] = (uint32_t)(((int64_t)(m - m0) * lda + ld_kc * 8) * 2);
         a_loff[i] = row * kRowBytes + swz(row, ld_kc) * 16;
     }
     if (B_NT) {
@@ -125,7 +128,7 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_reduce_kernel(const GemmArgs
     // descriptors: 48-bit base, stride 0 (raw), num_records 2^31-1 bytes, 32-bit data format.
     // Rows are clamped into the matrix above, so only the K tail needs the out-of-range path.
     const __amdgpu_buffer_rsrc_t a_rsrc =
-        __builtin_amdgcn_make_buffer_rsrc((void*)(g.A + (int64_t)m0 * g.lda), 0, 0x7fffffff, 0x00020000);
+        __builtin_amdgcn_make_buffer_rsrc((void*)a_tile, 0, 0x7fffffff, 0x00020000);
     const __amdgpu_buffer_rsrc_t bt_rsrc =
         __builtin_amdgcn_make_buffer_rsrc((void*)(g.B + (int64_t)n0 * g.ldb), 0, 0x7fffffff, 0x00020000);
 
@@ -364,13 +367,24 @@ static hipError_t launch_gemm(const GemmArgs& g, bool b_nt, bool even, hipStream
 
 using namespace kr;
 
-// Everything of the two entry points except the peers: argument checks in the documented
+// Arrival flags of the all-gather matmul (null pointer to gemm_reduce: A is complete).
+struct GatherSpec {
+    const void* a_local;
+    int64_t lda_local;
+    int64_t local_row0, local_rows;
+    const uint32_t* progress;
+    int64_t comm_rows;
+    int64_t wait_limit_us;
+    int* status;
+};
+
+// Everything of the entry points except the peers: argument checks in the documented
 // order, then tile choice and launch.  `peers_given` is the stacked base or the table.
 static int gemm_reduce(const void* A, int64_t lda_m, int64_t lda_k, const void* B, int64_t ldb_k, int64_t ldb_n,
                        int64_t M, int64_t N, int64_t K, const void* peers_given, int n_peers,
                        const void* const* peer_ptrs, int64_t peers_stride, const void* bias,
                        int64_t band_row0, int64_t band_rows, void* c_full, void* out, int out_is_fp32,
-                       int64_t tile_pivot, void* stream) {
+                       int64_t tile_pivot, void* stream, const GatherSpec* gather = nullptr) {
     if (M < 0 || N < 0 || K < 0 || M > 0x7fffffffLL || N > 0x7fffffffLL || K > 0x7fffffffLL)
         return KR_ERR_BAD_DIM;
     if (n_peers < 0 || n_peers >= KR_MAX_WORLD) return KR_ERR_WORLD_SIZE;
@@ -407,6 +421,23 @@ static int gemm_reduce(const void* A, int64_t lda_m, int64_t lda_k, const void* 
     g.ldb = ldb;
     g.M = (int)M; g.N = (int)N; g.K = (int)K;
     g.n_peers = n_peers;
+    g.progress = nullptr;
+    g.comm_rows = 1;
+    g.a_local = nullptr;
+    g.lda_local = 0;
+    g.local_row0 = g.local_rows = 0;
+    g.wait_ticks = 0;
+    g.status = nullptr;
+    if (gather != nullptr && gather->progress != nullptr) {
+        g.progress = gather->progress;
+        g.comm_rows = (int)gather->comm_rows;
+        g.a_local = (const uint16_t*)gather->a_local;
+        g.lda_local = gather->lda_local;
+        g.local_row0 = (int)gather->local_row0;
+        g.local_rows = (int)gather->local_rows;
+        g.wait_ticks = (uint64_t)gather->wait_limit_us * 100u;   // 100 MHz constant clock
+        g.status = gather->status;
+    }
     g.bias = (const uint16_t*)bias;
     g.band_row0 = (int)band_row0;
     g.band_rows = (int)band_rows;
@@ -424,7 +455,8 @@ static int gemm_reduce(const void* A, int64_t lda_m, int64_t lda_k, const void* 
         if (t[0] == '1') big = false;
         if (t[0] == '2') big = true;
     }
-    const bool dtl = big && gemm_dtl_supported(g);
+    const bool dtl = big && gemm_dtl_supported(g) &&
+                     (g.a_local == nullptr || (int64_t)256 * g.lda_local * 2 < 0x7fffffffLL);
     // KRAKEN_AMD_GEMM_PEERS=epilogue keeps the peers' partial sums out of the matrix cores
     // (they are then added in the epilogue, where a non-finite value stays in its element)
     g.peers_on_mfma = 1;
@@ -438,6 +470,11 @@ static int gemm_reduce(const void* A, int64_t lda_m, int64_t lda_k, const void* 
     // stream the peers' partial sums (HBM-bound), 16 lets neighbouring CUs read longer runs of
     // the same rows at about the same time.
     g.group_n = (n_peers > 0 && band_rows * 2 >= M) ? 16 : 8;
+    // Rows that arrive while the kernel runs: narrow groups, so that the range of tiles each XCD
+    // walks spans all row blocks in the order of their arrival (every XCD then starts on the
+    // local shard and waits little); with wide groups the XCDs that own the last blocks idle
+    // until those have arrived.
+    if (g.progress != nullptr) g.group_n = (g.tiles_n + kXcds - 1) / kXcds;
     if (const char* t = getenv("KRAKEN_AMD_GEMM_GROUP")) {
         const int v = atoi(t);
         if (v >= 1 && v <= 64) g.group_n = v;
@@ -469,4 +506,30 @@ extern "C" int kr_gemm_reduce_ptrs_bf16(const void* A, int64_t lda_m, int64_t ld
     return gemm_reduce(A, lda_m, lda_k, B, ldb_k, ldb_n, M, N, K, peers, n_peers,
                        peers != nullptr ? peers : kNoPeers, 0, bias, band_row0, band_rows, c_full, out,
                        out_is_fp32, tile_pivot, stream);
+}
+
+extern "C" int kr_all_gather_matmul_bf16(const void* A, int64_t lda_m, const void* A_local, int64_t lda_local,
+                                         const void* B, int64_t ldb_k, int64_t ldb_n, int64_t M, int64_t N,
+                                         int64_t K, int W, int rank, int splits_per_rank,
+                                         const uint32_t* progress, int64_t wait_limit_us, int32_t* status,
+                                         void* C, void* stream) {
+    if (W < 1 || W > KR_MAX_WORLD) return KR_ERR_WORLD_SIZE;
+    if (rank < 0 || rank >= W || splits_per_rank < 1) return KR_ERR_STRIPE;
+    if (M < 0 || M % ((int64_t)W * splits_per_rank) != 0) return KR_ERR_BAND;
+    if (A_local != nullptr && (!aligned16(A_local) || lda_local % 8 != 0)) return KR_ERR_ALIGNMENT;
+    if (A_local != nullptr && lda_local < K) return KR_ERR_LAYOUT;
+    if ((reinterpret_cast<uintptr_t>(progress) & 3u) != 0 || (reinterpret_cast<uintptr_t>(status) & 3u) != 0)
+        return KR_ERR_ALIGNMENT;
+    GatherSpec gs;
+    gs.a_local = A_local;
+    gs.lda_local = lda_local;
+    gs.local_rows = M / W;
+    gs.local_row0 = gs.local_rows * rank;
+    gs.progress = progress;
+    gs.comm_rows = M > 0 ? M / ((int64_t)W * splits_per_rank) : 1;
+    gs.wait_limit_us = wait_limit_us > 0 ? wait_limit_us : 5000000;   // 5 s
+    gs.status = status;
+    // no reduce: the band is every row, no peers, no bias; tile order rotated to the local shard
+    return gemm_reduce(A, lda_m, 1, B, ldb_k, ldb_n, M, N, K, nullptr, 0, nullptr, 0, nullptr, 0, M, nullptr, C, 0,
+                       gs.local_row0, stream, &gs);
 }

@@ -22,6 +22,14 @@ struct GemmArgs {
     int out_is_fp32;
     int pivot_tiles;   // rotation of the M-tile order
     int tiles_m, tiles_n;
+    // all-gather matmul with arrival flags (progress == nullptr: A is complete, nothing waits)
+    const uint32_t* progress;   // progress[b] == 1 once rows [b*comm_rows, (b+1)*comm_rows) of A have arrived
+    int comm_rows;
+    const uint16_t* a_local;    // this rank's own shard, rows [local_row0, local_row0+local_rows) of A: never waits
+    int64_t lda_local;
+    int local_row0, local_rows;
+    uint64_t wait_ticks;        // bound of one tile's wait, in ticks of the 100 MHz constant clock
+    int* status;                // set to 1 + block index by a tile whose wait ran out (may be nullptr)
     int group_n;         // column panels per scheduling group (tile_schedule)
     int peers_on_mfma;   // 256x256 kernel: add whole-band tiles' peers through the matrix cores
 };
@@ -31,6 +39,49 @@ bool gemm_dtl_supported(const GemmArgs& g);
 hipError_t launch_gemm_dtl(const GemmArgs& g, bool b_nt, hipStream_t st);
 
 constexpr int kXcds = 8;
+
+// A operand of the tile that starts at row m0 (bm rows), for the all-gather matmul: rows arrive
+// in blocks of g.comm_rows while the kernel runs, each block's flag in g.progress set to 1 by a
+// stream-ordered write behind its copy (kraken/fused/all_gather_matmul.py:95-110: a tile of
+// the local shard reads the shard itself, any other tile waits for its block's flag).  Called by
+// every wave of the workgroup: each polls the flags of the blocks the tile covers with
+// device-scope loads and a short sleep, then an acquire fence orders its own loads behind the
+// flag (so no workgroup barrier is needed); the wait is bounded (g.wait_ticks): a tile whose flag does not come records
+// 1 + block in g.status and goes on (its result is then meaningless), and later tiles see
+// the status and do not wait at all, so the grid always drains.
+__device__ __forceinline__ void gathered_a_tile(const GemmArgs& g, int m0, int bm, const uint16_t*& a_tile,
+                                                int64_t& lda) {
+    a_tile = g.A + (int64_t)m0 * g.lda;
+    lda = g.lda;
+    if (g.progress == nullptr) return;
+    const int m1 = min(m0 + bm, g.M);
+    if (g.a_local != nullptr && m0 >= g.local_row0 && m1 <= g.local_row0 + g.local_rows) {
+        a_tile = g.a_local + (int64_t)(m0 - g.local_row0) * g.lda_local;
+        lda = g.lda_local;
+        return;
+    }
+    const int b_hi = (m1 - 1) / g.comm_rows;
+    const uint64_t t0 = __builtin_amdgcn_s_memrealtime();
+    bool give_up = g.status != nullptr && __hip_atomic_load(g.status, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0;
+    for (int b = m0 / g.comm_rows; b <= b_hi && !give_up; ++b) {
+        while (__hip_atomic_load(g.progress + b, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 1u) {
+            if (__builtin_amdgcn_s_memrealtime() - t0 > g.wait_ticks) {
+                give_up = true;
+                if (g.status != nullptr) __hip_atomic_store(g.status, b + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                break;
+            }
+            __builtin_amdgcn_s_sleep(16);
+        }
+    }
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+}
+
+// a value every lane of the wave holds, moved to scalar registers
+__device__ __forceinline__ int64_t wave_uniform(int64_t v) {
+    const uint32_t lo = __builtin_amdgcn_readfirstlane((int)(uint32_t)v);
+    const uint32_t hi = __builtin_amdgcn_readfirstlane((int)(uint32_t)((uint64_t)v >> 32));
+    return (int64_t)(((uint64_t)hi << 32) | lo);
+}
 
 // Map the workgroup id to its tile (tile_m, tile_n).
 __device__ __forceinline__ void tile_schedule(const GemmArgs& g, int& tile_m_out, int& tile_n_out) {

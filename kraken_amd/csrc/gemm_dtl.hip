@@ -74,6 +74,13 @@ __device__ __forceinline__ void gemm_dtl_tile(const GemmArgs& g, unsigned char* 
     int tile_m, tile_n;
     tile_schedule(g, tile_m, tile_n);
     const int m0 = tile_m * BM, n0 = tile_n * BN;
+    const uint16_t* a_tile;   // first row of the tile's A panel (gathered matrix or local shard)
+    int64_t lda;
+    gathered_a_tile(g, m0, BM, a_tile, lda);
+    // (the choice above is the same for the whole workgroup; the descriptor below wants it in
+    // scalar registers)
+    a_tile = (const uint16_t*)wave_uniform((int64_t)a_tile);
+    lda = wave_uniform(lda);
 
     // ---- LDS-DMA addressing ----------------------------------------------------------------
     // A wave loads the 1 KiB chunks  wave, wave+4, ..., wave+28  of a stage.
@@ -82,7 +89,7 @@ __device__ __forceinline__ void gemm_dtl_tile(const GemmArgs& g, unsigned char* 
     // has the parity of the wave, so the per-lane byte offset is computed once; the wave-uniform
     // part (chunk row, k) goes to the scalar offset.
     const int dma_sw = (4 * (wave & 1) + (lane >> 4)) & 7;
-    const uint32_t a_voff_lane = (uint32_t)(((int64_t)(lane >> 3) * g.lda + (((lane & 7) ^ dma_sw) << 3)) * 2);
+    const uint32_t a_voff_lane = (uint32_t)(((int64_t)(lane >> 3) * lda + (((lane & 7) ^ dma_sw) << 3)) * 2);
     uint32_t b_voff_lane;
     if (B_NT) {
         b_voff_lane = (uint32_t)(((int64_t)(lane >> 3) * g.ldb + (((lane & 7) ^ dma_sw) << 3)) * 2);
@@ -116,7 +123,7 @@ __device__ __forceinline__ void gemm_dtl_tile(const GemmArgs& g, unsigned char* 
                      : "s"(lds_addr), "v"(voff), "s"(rsrc), "s"(soff)
                      : "memory", "m0");
     };
-    const i32x4 a_rsrc = make_rsrc(g.A + (int64_t)m0 * g.lda);
+    const i32x4 a_rsrc = make_rsrc(a_tile);
     const i32x4 bt_rsrc = make_rsrc(g.B + (int64_t)n0 * g.ldb);
 
     const int kt_total = g.K / BKD;
@@ -131,7 +138,7 @@ __device__ __forceinline__ void gemm_dtl_tile(const GemmArgs& g, unsigned char* 
         const uint32_t a_voff = live ? a_voff_lane : 0u, b_voff = live ? b_voff_lane : 0u;
         const int ch = wave + 4 * (q % LOADS_A);
         if (q < LOADS_A) {
-            lds_dma_b128(a_rsrc, stage * A_ST + ch * 1024, a_voff, (int)(((int64_t)8 * ch * g.lda + k0) * 2));
+            lds_dma_b128(a_rsrc, stage * A_ST + ch * 1024, a_voff, (int)(((int64_t)8 * ch * lda + k0) * 2));
         } else if (B_NT) {
             lds_dma_b128(bt_rsrc, B_BASE + stage * B_ST + ch * 1024, b_voff,
                          (int)(((int64_t)8 * ch * g.ldb + k0) * 2));

@@ -3,11 +3,43 @@ from __future__ import annotations
 
 import torch
 
+from .. import _lib
+from ..comm._common import PeerBuffers
+from ..comm.copy_engine_all_gather import _copy_engine_all_gather_w_progress
 from . import _gemm
 
 
+def _matmul_w_progress(a, a_local, b, progress, configs, status=None) -> torch.Tensor:
+    """``c = a @ b`` where the rows of ``a`` arrive while the kernel runs.
+
+    Counterpart of ``_matmul_w_progress`` (``kraken/fused/all_gather_matmul.py:147-219``):
+    tiles of the local shard read ``a_local``, all others wait for
+    ``progress[chunk] == 1`` (``:95-110``).  ``configs``: ``RANK``, ``WORLD_SIZE``,
+    ``SPLITS_PER_RANK``, optional ``wait_limit_us``.
+    """
+    M, K = a.shape
+    assert b.shape[0] == K
+    if not b.T.is_contiguous():
+        raise ValueError("b.T must be contiguous")
+    N = b.shape[1]
+    assert K % 8 == 0 and N % 8 == 0, "K and N must be multiples of 8"
+    assert a.dtype == torch.bfloat16 and b.dtype == torch.bfloat16, "Only bfloat16 is supported for now."
+    assert a.stride(1) == 1 and (a_local is None or a_local.stride(1) == 1)
+    dev = _lib.require_device(a, a_local, b, progress, status)
+    c = torch.empty((M, N), device=dev, dtype=a.dtype)
+    rc = _lib.load().kr_all_gather_matmul_bf16(
+        a.data_ptr(), a.stride(0), _lib.ptr(a_local), 0 if a_local is None else a_local.stride(0),
+        b.data_ptr(), b.stride(0), b.stride(1), M, N, K,
+        configs["WORLD_SIZE"], configs["RANK"], configs["SPLITS_PER_RANK"],
+        _lib.ptr(progress), int(configs.get("wait_limit_us", 0)), _lib.ptr(status),
+        c.data_ptr(), _lib.current_stream(dev),
+    )
+    _lib.check(rc, "all_gather_matmul")
+    return c
+
+
 def all_gather_matmul(
-    a_shared: torch.Tensor,
+    a_shared,
     b: torch.Tensor,
     a_out: torch.Tensor | None = None,
     progress: torch.Tensor | None = None,
@@ -17,36 +49,74 @@ def all_gather_matmul(
 
     Counterpart of ``kraken.fused.all_gather_matmul``
     (``kraken/fused/all_gather_matmul.py:222-325``; arithmetic ``:87-123``).
-    ``a_shared`` is the ``[W, m, K]`` stack of all ranks' shards — already
-    "gathered" on one GPU — so ``a_gathered`` is its zero-copy ``[W*m, K]``
-    view (copied into ``a_out`` when one is passed).  ``b`` must satisfy
-    ``b.T.is_contiguous()`` like in the reference (``:158-160``).  The order of
-    the M tiles is rotated so that the shard of ``rank`` (kwarg, default 0) is
-    consumed first (``:93``); this changes scheduling only.  ``progress``, if
-    given, is set to 1 everywhere (all chunks present).  Tile-size kwargs
-    (``splits_per_rank``, ``block_size_*``, ``group_size_m``, ``num_stages``,
-    ``num_warps``) are accepted and ignored.
+    ``a_shared`` holds all ranks' shards: the ``[W, m, K]`` stack or a list of
+    W separate ``[m, K]`` tensors.  ``b`` must satisfy ``b.T.is_contiguous()``
+    like in the reference (``:158-160``).  Two modes (kwarg ``gather``):
+
+    * ``gather=False`` (default for a contiguous stack): the stack already is
+      the gathered matrix, so ``a_gathered`` is its zero-copy ``[W*m, K]`` view
+      (copied into ``a_out`` when one is passed), ``progress`` is set to 1
+      everywhere and the GEMM waits for nothing.
+    * ``gather=True`` (default for a list of shards): the reference's overlap.
+      The shards are copied chunk by chunk into ``a_out`` on a side stream,
+      each chunk followed by its flag in ``progress`` (``:308-311``), while the
+      GEMM on the current stream consumes them: tiles of the local shard
+      (``rank``) read it in place, every other tile waits for its chunk's flag
+      (``:95-110``).  The current stream then waits for the side stream
+      (``:316``).  ``status`` (int32 ``[1]``, zeroed by the caller) receives a
+      non-zero value if a tile's wait ran out (``wait_limit_us``, default 5 s).
+
+    In both modes the order of the M tiles is rotated so that the shard of
+    ``rank`` (kwarg, default 0) is consumed first and the others in the order
+    the copies are issued (``:93``).  ``splits_per_rank`` (default 1) chunks per
+    shard; the remaining tile-size kwargs are accepted and ignored.
     """
-    assert a_shared.dim() == 3, "expected the stacked shards [W, m, K]"
-    assert a_shared.dtype == torch.bfloat16 and b.dtype == torch.bfloat16, "Only bfloat16 is supported for now."
-    assert a_shared.is_contiguous()
-    W, m, K = a_shared.shape
+    peers = PeerBuffers(a_shared)
+    W = peers.W
+    shard = peers.slice(0)
+    assert shard.dim() == 2, "expected shards of shape [m, K]"
+    assert b.dtype == torch.bfloat16, "Only bfloat16 is supported for now."
+    m, K = shard.shape
     assert b.dim() == 2 and b.shape[0] == K
     if not b.T.is_contiguous():
         raise ValueError("b.T must be contiguous")
     rank = kwargs.get("rank", 0)
     assert 0 <= rank < W
-    a_full = a_shared.reshape(W * m, K)
-    if a_out is not None:
-        assert a_out.shape == a_full.shape and a_out.dtype == a_full.dtype
-        a_out.copy_(a_full)
-    else:
-        a_out = a_full
-    if progress is not None:
-        progress.fill_(1)
-    a2, b2 = _gemm.prepare_operands(a_full, b)
+    splits = kwargs.get("splits_per_rank", 1)
     M, N = W * m, b.shape[1]
     assert N % 8 == 0, "N must be a multiple of 8"
-    c = torch.empty((M, N), dtype=a_shared.dtype, device=a_shared.device)
-    _gemm.launch("all_gather_matmul", a2, b2, M, N, None, 0, 0, None, 0, M, None, c, rank * m)
+    stacked = peers.stacked is not None and peers.stacked.is_contiguous()
+    gather = kwargs.get("gather", not stacked)
+    dev = _lib.require_device(*peers.tensors, b, a_out, progress)
+
+    if not gather:
+        assert stacked, "gather=False needs the shards as one contiguous [W, m, K] tensor"
+        a_full = peers.stacked.reshape(M, K)
+        if a_out is not None:
+            assert a_out.shape == a_full.shape and a_out.dtype == a_full.dtype
+            a_out.copy_(a_full)
+        else:
+            a_out = a_full
+        if progress is not None:
+            progress.fill_(1)
+        a2, b2 = _gemm.prepare_operands(a_full, b)
+        c = torch.empty((M, N), dtype=torch.bfloat16, device=dev)
+        _gemm.launch("all_gather_matmul", a2, b2, M, N, None, 0, 0, None, 0, M, None, c, rank * m)
+        return a_out, c
+
+    assert K % 8 == 0, "K must be a multiple of 8"
+    assert m % splits == 0, "splits_per_rank must divide the rows of a shard"
+    if a_out is None:
+        a_out = torch.empty((M, K), dtype=torch.bfloat16, device=dev)
+    else:
+        assert tuple(a_out.shape) == (M, K) and a_out.dtype == torch.bfloat16 and a_out.is_contiguous()
+    if progress is None:
+        progress = torch.zeros(W * splits, dtype=torch.int32, device=dev)
+    else:
+        progress.fill_(0)
+    backend_stream = _copy_engine_all_gather_w_progress(a_out, a_shared, progress, splits, rank=rank)
+    configs = {"RANK": rank, "WORLD_SIZE": W, "SPLITS_PER_RANK": splits,
+               "wait_limit_us": kwargs.get("wait_limit_us", 0)}
+    c = _matmul_w_progress(a_out, peers.slice(rank), b, progress, configs, kwargs.get("status"))
+    torch.cuda.current_stream(dev).wait_stream(backend_stream)
     return a_out, c

@@ -159,6 +159,32 @@ def test_wrappers_accept_a_list_of_buffers_and_check_it():
         fused.gemm_one_shot_all_reduce_fused(a, b, peers=[torch.zeros(8, 8, dtype=BF16)])
 
 
+def test_all_gather_matmul_argument_errors(lib):
+    f = lib.kr_all_gather_matmul_bf16
+    def args(**kw):
+        a = dict(A=FAKE, lda_m=64, A_local=FAKE, lda_local=64, B=FAKE, ldb_k=1, ldb_n=64, M=512, N=64, K=64,
+                 W=4, rank=1, splits=2, progress=FAKE, wait_us=0, status=FAKE, C=FAKE, stream=None)
+        a.update(kw)
+        return tuple(a.values())
+    assert f(*args(W=0)) == _lib.KR_ERR_WORLD_SIZE
+    assert f(*args(W=17)) == _lib.KR_ERR_WORLD_SIZE
+    assert f(*args(rank=4)) == _lib.KR_ERR_STRIPE
+    assert f(*args(splits=0)) == _lib.KR_ERR_STRIPE
+    assert f(*args(M=500)) == _lib.KR_ERR_BAND             # 500 rows do not split into 4*2 chunks
+    assert f(*args(A_local=FAKE + 2)) == _lib.KR_ERR_ALIGNMENT
+    assert f(*args(lda_local=32)) == _lib.KR_ERR_LAYOUT      # shorter than K
+    assert f(*args(progress=FAKE + 2)) == _lib.KR_ERR_ALIGNMENT
+    assert f(*args(status=FAKE + 1)) == _lib.KR_ERR_ALIGNMENT
+    assert f(*args(A=None)) == _lib.KR_ERR_NULL_POINTER
+    assert f(*args(C=None)) == _lib.KR_ERR_NULL_POINTER
+    assert f(*args(K=60)) == _lib.KR_ERR_NUMEL_MOD8
+    assert f(*args(ldb_k=2, ldb_n=3)) == _lib.KR_ERR_LAYOUT
+    assert f(*args(M=0)) == 0
+    g = lib.kr_stream_write_value32
+    assert g(None, 1, None) == _lib.KR_ERR_NULL_POINTER
+    assert g(FAKE + 2, 1, None) == _lib.KR_ERR_ALIGNMENT
+
+
 def test_striped_share_numel(lib):
     f = lib.kr_striped_share_numel
     numel, W, block = 8 * 37, 4, 16
@@ -189,8 +215,9 @@ def test_check_maps_codes_to_reference_exceptions():
 
 
 def test_public_names_match_reference_layout():
-    # kraken/comm/__init__.py:12-17 (reduce entry points), kraken/fused/__init__.py:17-27
-    assert set(comm.__all__) == {"one_shot_all_reduce", "two_shot_all_reduce"}
+    # kraken/comm/__init__.py:12-17, kraken/fused/__init__.py:17-27
+    assert set(comm.__all__) == {"_copy_engine_all_gather_w_progress", "all_gather_w_progress",
+                                 "one_shot_all_reduce", "two_shot_all_reduce"}
     assert set(fused.__all__) == {
         "all_gather_matmul", "gemm_one_shot_all_reduce_fused", "gemm_reduce_scatter",
         "gemm_reduce_scatter_ce_persistent", "one_shot_all_reduce_bias",

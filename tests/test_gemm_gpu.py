@@ -5,7 +5,7 @@ import os
 import pytest
 import torch
 
-from kraken_amd import fused
+from kraken_amd import comm, fused
 from oracle import oracle as orc
 
 pytestmark = pytest.mark.gpu
@@ -121,6 +121,69 @@ def test_all_gather_matmul(dev, tile, rank):
     a_out = torch.empty(W * m, K, dtype=BF16, device=dev)
     ag2, c2 = fused.all_gather_matmul(sd, bT.to(dev).T, a_out=a_out, rank=rank)
     assert ag2 is a_out and torch.equal(a_out.cpu(), a_want) and torch.equal(c2, c)
+
+
+@pytest.mark.parametrize("rank,splits", [(0, 1), (2, 2), (3, 4)])
+@pytest.mark.parametrize("as_list", [False, True])
+def test_all_gather_matmul_overlapped_with_the_copies(dev, tile, rank, splits, as_list):
+    """The reference's overlap: chunk copies with arrival flags on a side stream, tiles that
+    wait for their chunk (kraken/fused/all_gather_matmul.py:95-110); local shard read in place."""
+    W, m, K, N = 4, 256, 320, 384
+    stack = orc.make_stack(W, (m, K), seed0=7)
+    bT = orc.randn_bf16((N, K), 43, 0.05)
+    a_want, c_want = orc.all_gather_matmul(stack, bT.T)
+    shards = [stack[r].to(dev) for r in range(W)] if as_list else stack.to(dev)
+    progress = torch.full((W * splits,), 7, dtype=torch.int32, device=dev)       # stale values: must be reset
+    status = torch.zeros(1, dtype=torch.int32, device=dev)
+    a_out = torch.full((W * m, K), float("nan"), dtype=BF16, device=dev)
+    ag, c = fused.all_gather_matmul(shards, bT.to(dev).T, a_out=a_out, progress=progress, rank=rank,
+                                    splits_per_rank=splits, gather=True, status=status)
+    torch.cuda.synchronize()
+    assert ag is a_out and torch.equal(ag.cpu(), a_want)          # test/test_allgather_matmul.py:75: exact
+    assert (progress == 1).all()                                  # test/test_allgather.py:73
+    assert status.item() == 0
+    torch.testing.assert_close(c.cpu(), c_want, **TOL)
+    # same bits as the GEMM on the already gathered matrix
+    _, c_plain = fused.all_gather_matmul(stack.to(dev), bT.to(dev).T, rank=rank)
+    assert torch.equal(c, c_plain)
+
+
+def test_all_gather_w_progress(dev):
+    # test/test_allgather.py:50-75: gathered tensor exact, every flag set
+    W, m, K = 8, 64, 128
+    stack = orc.make_stack(W, (m, K), seed0=3)
+    for splits, rank in ((1, 0), (4, 5)):
+        progress = torch.zeros(W * splits, dtype=torch.int32, device=dev)
+        out = comm.all_gather_w_progress([stack[r].to(dev) for r in range(W)], progress=progress,
+                                         splits_per_rank=splits, rank=rank)
+        torch.cuda.synchronize()
+        assert torch.equal(out.cpu(), stack.reshape(W * m, K))
+        assert (progress == 1).all()
+
+
+def test_all_gather_matmul_wait_is_bounded(dev, tile):
+    """A flag that never comes: every tile's wait ends at the limit, the kernel exits and the
+    status names a chunk (no copy is enqueued here; the limit is 2 ms)."""
+    from kraken_amd.fused.all_gather_matmul import _matmul_w_progress
+    W, m, K, N = 4, 256, 128, 256
+    a = orc.randn_bf16((W * m, K), 1).to(dev)
+    bT = orc.randn_bf16((N, K), 2, 0.05).to(dev)
+    progress = torch.zeros(W, dtype=torch.int32, device=dev)
+    progress[1] = 1                                               # one chunk present, two missing
+    status = torch.zeros(1, dtype=torch.int32, device=dev)
+    cfg = {"RANK": 0, "WORLD_SIZE": W, "SPLITS_PER_RANK": 1, "wait_limit_us": 2000}
+    c = _matmul_w_progress(a, a[:m], bT.T, progress, cfg, status)
+    torch.cuda.synchronize()
+    assert status.item() in (3, 4)                                # 1 + index of a missing chunk
+    want = (a.float().cpu() @ bT.float().cpu().T).to(BF16)
+    torch.testing.assert_close(c[:2 * m].cpu(), want[:2 * m], **TOL)   # local shard and the present chunk
+    # with every flag set the same call is complete and the status stays clear
+    progress.fill_(1)
+    status.zero_()
+    c = _matmul_w_progress(a, a[:m], bT.T, progress, cfg, status)
+    torch.cuda.synchronize()
+    assert status.item() == 0
+    torch.testing.assert_close(c.cpu(), want, **TOL)
 
 
 def test_ce_persistent_variant(dev, tile):
