@@ -479,6 +479,16 @@ def main() -> None:
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="instead of a workload, run plain device copies of 256 MiB (a kernel of known "
                          "traffic: 268435456 B read + 268435456 B written per launch) to scale profiler counters")
+    ap.add_argument("--sweep", default=None,
+                    choices=["all_reduce", "all_reduce_bias", "all_reduce_bias_rms_norm", "matmul_reduce_scatter",
+                             "all_gather_matmul"],
+                    help="instead of the JSON line, sweep shapes and print a backend table like the reference's "
+                         "benchmark/benchmark_*.py (first backend = baseline)")
+    ap.add_argument("--backend", nargs="+", default=None, help="--sweep: backends to compare (default: all)")
+    ap.add_argument("--shape", nargs="+", default=None,
+                    help="--sweep: shapes, comma separated (e.g. 1024,6656,8192; a single number for all_reduce)")
+    ap.add_argument("--world-size", type=int, default=8, help="--sweep: number of ranks whose buffers are reduced")
+    ap.add_argument("--save-path", default=None, help="--sweep: also write the table as CSV")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         _die_multi_gpu(max(args.gpus, int(os.environ.get("WORLD_SIZE", "1"))))
@@ -494,6 +504,17 @@ def main() -> None:
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
     threads = torch.get_num_threads()
+
+    if args.sweep:
+        from kraken_amd._logging.sweep import run_sweep
+
+        shapes = None
+        if args.shape:
+            shapes = [tuple(int(x) for x in sh.split(",")) for sh in args.shape]
+            if args.sweep == "all_reduce":
+                shapes = [sh[0] for sh in shapes]
+        run_sweep(args.sweep, args.backend, shapes, args.world_size, args.save_path, dev=dev)
+        return
 
     if args.calibrate_copy:
         src = torch.empty(128 * 1024 * 1024, dtype=torch.bfloat16, device=dev).normal_()
