@@ -206,6 +206,41 @@ int kr_gemm_reduce_ptrs_bf16(const void* A, int64_t lda_m, int64_t lda_k,
                              int64_t tile_pivot, void* stream);
 
 /*
+ * kr_gemm_reduce_bf16 / kr_gemm_reduce_ptrs_bf16 with a workspace, for shapes with few output
+ * tiles (few rows: M of a few hundred) whose K loop is then split over S workgroups per tile so
+ * that all CUs have work.  Two launches: the S partial products go to the workspace in fp32; a
+ * second kernel sums them in the order 0..S-1 and applies the epilogue (peers, bias, band, c_full)
+ * with the adds in the same order and the same rounding as the one-pass kernel.  Results are
+ * reproducible run to run and differ from the unsplit result only by the fp32 rounding of the
+ * order in which the k-steps are summed.  `workspace`: device memory, 16-byte aligned, of at
+ * least kr_gemm_workspace_bytes(M, N, K) bytes (0: this shape is not split); its contents
+ * before the call do not matter and are undefined after it.  Calls that use one workspace must
+ * not overlap (same stream, or otherwise ordered).  workspace == NULL, a workspace that is too
+ * small, or a shape that does not profit: exactly the entry point without workspace.
+ * No counterpart in the reference (its GEMM kernels launch one program per output tile,
+ * kraken/fused/gemm_reduce_scatter_fused.py:202-204, gemm_one_shot_all_reduce_fused.py:149-153).
+ */
+int64_t kr_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K);
+int kr_gemm_reduce_ws_bf16(const void* A, int64_t lda_m, int64_t lda_k,
+                           const void* B, int64_t ldb_k, int64_t ldb_n,
+                           int64_t M, int64_t N, int64_t K,
+                           const void* peers, int n_peers, int64_t peers_stride,
+                           const void* bias,
+                           int64_t band_row0, int64_t band_rows,
+                           void* c_full, void* out, int out_is_fp32,
+                           int64_t tile_pivot,
+                           void* workspace, int64_t workspace_bytes, void* stream);
+int kr_gemm_reduce_ptrs_ws_bf16(const void* A, int64_t lda_m, int64_t lda_k,
+                                const void* B, int64_t ldb_k, int64_t ldb_n,
+                                int64_t M, int64_t N, int64_t K,
+                                const void* const* peers, int n_peers,
+                                const void* bias,
+                                int64_t band_row0, int64_t band_rows,
+                                void* c_full, void* out, int out_is_fp32,
+                                int64_t tile_pivot,
+                                void* workspace, int64_t workspace_bytes, void* stream);
+
+/*
  * All-gather matmul that consumes A while it is still arriving:  C[M,N] = A[M,K] @ B[K,N]  (bf16, fp32
  * accumulate, bf16 result), where A is the gathered matrix of W shards of M/W rows, filled by
  * copies that run on another stream while this kernel runs.  The rows arrive in W*splits_per_rank

@@ -61,6 +61,19 @@ _SIGNATURES = {
         [c_void_p, c_int64, c_int64, c_void_p, c_int64, c_int64, c_int64, c_int64, c_int64,
          c_void_p, c_int, c_int64, c_void_p, c_int64, c_int64, c_void_p, c_void_p, c_int, c_int64, c_void_p],
     ),
+    "kr_gemm_workspace_bytes": (c_int64, [c_int64, c_int64, c_int64]),
+    "kr_gemm_reduce_ws_bf16": (
+        c_int,
+        [c_void_p, c_int64, c_int64, c_void_p, c_int64, c_int64, c_int64, c_int64, c_int64,
+         c_void_p, c_int, c_int64, c_void_p, c_int64, c_int64, c_void_p, c_void_p, c_int, c_int64,
+         c_void_p, c_int64, c_void_p],
+    ),
+    "kr_gemm_reduce_ptrs_ws_bf16": (
+        c_int,
+        [c_void_p, c_int64, c_int64, c_void_p, c_int64, c_int64, c_int64, c_int64, c_int64,
+         c_void_p, c_int, c_void_p, c_int64, c_int64, c_void_p, c_void_p, c_int, c_int64,
+         c_void_p, c_int64, c_void_p],
+    ),
     "kr_all_gather_matmul_bf16": (
         c_int,
         [c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_int64, c_int64, c_int64, c_int64, c_int64,

@@ -23,6 +23,8 @@
 
 #include <type_traits>
 
+#include <algorithm>
+
 #include "gemm_common.h"
 
 namespace kr {
@@ -72,6 +74,12 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_reduce_kernel(const GemmArgs
     const uint16_t* a_tile;   // first row of the tile's A panel (gathered matrix or local shard)
     int64_t lda;
     gathered_a_tile(g, m0, BM, a_tile, lda);
+    // k range of this workgroup: all of K, or with a split K loop (g.k_splits > 1, split index
+    // in blockIdx.y) the split's share of the k-steps; k_begin enters every operand offset
+    const int kt_all = (g.K + BK - 1) / BK;
+    const int kt_begin = g.k_splits > 1 ? (int)((int64_t)kt_all * blockIdx.y / g.k_splits) : 0;
+    const int kt_total = g.k_splits > 1 ? (int)((int64_t)kt_all * (blockIdx.y + 1) / g.k_splits) - kt_begin : kt_all;
+    const int k_begin = kt_begin * BK;
 
     f32x16 acc[TM][TN];
 #pragma unroll
@@ -132,12 +140,14 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_reduce_kernel(const GemmArgs
     const __amdgpu_buffer_rsrc_t bt_rsrc =
         __builtin_amdgcn_make_buffer_rsrc((void*)(g.B + (int64_t)n0 * g.ldb), 0, 0x7fffffff, 0x00020000);
 
-    auto load_a_unit = [&](int rs, int i, int k0) {
+    auto load_a_unit = [&](int rs, int i, int k_rel) {
+        const int k0 = k_begin + k_rel;
         uint32_t off = a_goff[i];
         if (!EVEN && k0 + ld_kc * 8 >= g.K) off = kOob;
         a_reg[rs][i] = __builtin_amdgcn_raw_buffer_load_b128(a_rsrc, off, k0 * 2, 0);
     };
-    auto load_b_unit = [&](int rs, int u, int k0) {
+    auto load_b_unit = [&](int rs, int u, int k_rel) {
+        const int k0 = k_begin + k_rel;
         if (B_NT) {
             uint32_t off = b_goff[u];
             if (!EVEN && k0 + ld_kc * 8 >= g.K) off = kOob;
@@ -214,7 +224,6 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_reduce_kernel(const GemmArgs
     // issued (and waited for) its last reads of tile t.  All side work is spread between the
     // MFMAs in a fixed order.
     constexpr int NM = TM * TN, NF = TM + TN;
-    const int kt_total = (g.K + BK - 1) / BK;
     const int k_last = (kt_total - 1) * BK;
 
 #define KR_SCHED_FENCE() __builtin_amdgcn_sched_barrier(0)
@@ -337,11 +346,49 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_reduce_kernel(const GemmArgs
     gemm_epilogue<BM, WTM, WTN, TM, TN, EVEN, EP_WAVE>(g, g.n_peers, g.bias, acc, smem, m0, n0, wm, wn, lane, wave);
 }
 
+// Second pass of the split K loop: sums the S fp32 partial products [S][M][N] in the order
+// 0..S-1 and applies the epilogue of the one-pass kernel (same order of the adds, same
+// rounding: with a bf16 result and peers the product is rounded to bf16 before the peers'
+// partial sums are added).  One thread per 8 consecutive columns.
+__global__ __launch_bounds__(256) void splitk_finish_kernel(const GemmArgs g, const float* __restrict__ parts, int S) {
+    const int64_t v = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    const int nv = g.N / 8;
+    if (v >= (int64_t)g.M * nv) return;
+    const int m = (int)(v / nv), n = (int)(v - (int64_t)m * nv) * 8;
+    const int64_t mn = (int64_t)g.M * g.N;
+    const float* p = parts + (int64_t)m * g.N + n;
+    float f[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) f[j] = 0.0f;
+    for (int sp = 0; sp < S; ++sp) {
+        const f32x4 lo = __builtin_nontemporal_load((const f32x4*)(p + sp * mn));
+        const f32x4 hi = __builtin_nontemporal_load((const f32x4*)(p + sp * mn + 4));
+        f[0] += lo.x; f[1] += lo.y; f[2] += lo.z; f[3] += lo.w;
+        f[4] += hi.x; f[5] += hi.y; f[6] += hi.z; f[7] += hi.w;
+    }
+    const int mb = m - g.band_row0;
+    if (mb < 0 || mb >= g.band_rows) {
+        if (g.c_full != nullptr) st_stream((u32x4*)(g.c_full + (int64_t)m * g.N + n), pack8(f));
+        return;
+    }
+    const int64_t off = (int64_t)mb * g.N + n;
+    if (!g.out_is_fp32 && g.n_peers > 0) unpack8(pack8(f), f);
+    for (int q = 0; q < g.n_peers; ++q) add8(ld_stream((const u32x4*)((const uint16_t*)g.peer.p[q] + off)), f);
+    if (g.bias != nullptr) add8(*(const u32x4*)(g.bias + n), f);
+    if (g.out_is_fp32) {
+        float* o = (float*)g.out + off;
+        *(f32x4*)o = f32x4{f[0], f[1], f[2], f[3]};
+        *(f32x4*)(o + 4) = f32x4{f[4], f[5], f[6], f[7]};
+    } else {
+        st_stream((u32x4*)((uint16_t*)g.out + off), pack8(f));
+    }
+}
+
 template <int BM, int BN, int WM, int WN>
 static hipError_t launch_gemm(const GemmArgs& g, bool b_nt, bool even, hipStream_t st) {
     constexpr int T = WM * WN * 64;
     constexpr int LDS = 2 * (BM + BN) * kRowBytes;
-    const dim3 grid((unsigned)(g.tiles_m * g.tiles_n)), block(T);
+    const dim3 grid((unsigned)(g.tiles_m * g.tiles_n), (unsigned)g.k_splits), block(T);
 #define KR_LAUNCH(NT, EV)                                                                             \
     do {                                                                                              \
         auto kfn = gemm_reduce_kernel<BM, BN, WM, WN, NT, EV>;                                        \
@@ -367,6 +414,27 @@ static hipError_t launch_gemm(const GemmArgs& g, bool b_nt, bool even, hipStream
 
 using namespace kr;
 
+// ---- split K loop: how many workgroups share a tile ------------------------------------------
+// A tile's K loop is split when the tiles alone leave CUs empty: into as many parts as fill the
+// 256 CUs once (measured on M = 128..1024, N = 6656, K = 4096 and 16384: 52 tiles -> 4 parts,
+// 104 -> 2, 208 and more -> 1 were the fastest or within a few percent of it; more parts only
+// add partial products to write and read), each with at least kMinSplitSteps k-steps of 64.
+constexpr int kMaxSplits = 16;
+constexpr int kMinSplitSteps = 8;
+static int split_k_factor(int64_t tiles, int64_t K) {
+    if (const char* t = getenv("KRAKEN_AMD_GEMM_SPLITK")) {   // testing and tuning
+        const int v = atoi(t);
+        if (v >= 1 && v <= kMaxSplits) return (int)std::min<int64_t>(v, std::max<int64_t>(1, (K + BK - 1) / BK));
+    }
+    if (tiles <= 0 || tiles * 2 > 256) return 1;
+    int64_t s = 256 / tiles;
+    s = std::min<int64_t>(s, ((K + BK - 1) / BK) / kMinSplitSteps);
+    s = std::min<int64_t>(s, kMaxSplits);
+    return (int)std::max<int64_t>(s, 1);
+}
+// workspace of the two-pass form: S fp32 partial products of the whole [M, N] result
+static int64_t split_k_workspace_bytes(int64_t M, int64_t N, int S) { return (int64_t)S * M * N * 4; }
+
 // Arrival flags of the all-gather matmul (null pointer to gemm_reduce: A is complete).
 struct GatherSpec {
     const void* a_local;
@@ -384,7 +452,8 @@ static int gemm_reduce(const void* A, int64_t lda_m, int64_t lda_k, const void* 
                        int64_t M, int64_t N, int64_t K, const void* peers_given, int n_peers,
                        const void* const* peer_ptrs, int64_t peers_stride, const void* bias,
                        int64_t band_row0, int64_t band_rows, void* c_full, void* out, int out_is_fp32,
-                       int64_t tile_pivot, void* stream, const GatherSpec* gather = nullptr) {
+                       int64_t tile_pivot, void* stream, const GatherSpec* gather = nullptr,
+                       void* workspace = nullptr, int64_t workspace_bytes = 0) {
     if (M < 0 || N < 0 || K < 0 || M > 0x7fffffffLL || N > 0x7fffffffLL || K > 0x7fffffffLL)
         return KR_ERR_BAD_DIM;
     if (n_peers < 0 || n_peers >= KR_MAX_WORLD) return KR_ERR_WORLD_SIZE;
@@ -481,9 +550,38 @@ static int gemm_reduce(const void* A, int64_t lda_m, int64_t lda_k, const void* 
         const int v = atoi(t);
         if (v >= 1 && v <= 64) g.group_n = v;
     }
+    // Split K loop (128x128 kernel, workspace given): with few tiles most CUs would idle, so S
+    // workgroups share a tile's K loop and meet in the workspace.
+    g.k_splits = 1;
+    g.split_out_stride = 0;
+    int splits = 1;
+    if (!dtl && workspace != nullptr) {
+        splits = split_k_factor((int64_t)g.tiles_m * g.tiles_n, K);
+        if (splits > 1 && split_k_workspace_bytes(M, N, splits) > workspace_bytes) splits = 1;
+        if (splits > 1 && !aligned16(workspace)) return KR_ERR_ALIGNMENT;
+    }
     int64_t pt = tile_pivot / bm;
     g.pivot_tiles = (int)(((pt % g.tiles_m) + g.tiles_m) % g.tiles_m);
     const bool even = (M % bm == 0 && N % bn == 0 && K % BK == 0);
+    if (splits > 1) {
+        // pass 1: S partial products, fp32, no epilogue work; pass 2: sum + epilogue
+        GemmArgs g1 = g;
+        g1.k_splits = splits;
+        g1.split_out_stride = M * N;
+        g1.out = workspace;
+        g1.out_is_fp32 = 1;
+        g1.n_peers = 0;
+        g1.bias = nullptr;
+        g1.band_row0 = 0;
+        g1.band_rows = (int)M;
+        g1.c_full = nullptr;
+        hipError_t e = launch_gemm<128, 128, 2, 2>(g1, b_nt, even, (hipStream_t)stream);
+        if (e != hipSuccess) return (int)e;
+        const int64_t vecs = M * (N / 8);
+        hipLaunchKernelGGL(splitk_finish_kernel, dim3((unsigned)((vecs + 255) / 256)), dim3(256), 0,
+                           (hipStream_t)stream, g, (const float*)workspace, splits);
+        return (int)hipGetLastError();
+    }
     hipError_t e = dtl ? launch_gemm_dtl(g, b_nt, (hipStream_t)stream)
                        : launch_gemm<128, 128, 2, 2>(g, b_nt, even, (hipStream_t)stream);
     return (int)e;
@@ -534,4 +632,34 @@ extern "C" int kr_all_gather_matmul_bf16(const void* A, int64_t lda_m, const voi
     // no reduce: the band is every row, no peers, no bias; tile order rotated to the local shard
     return gemm_reduce(A, lda_m, 1, B, ldb_k, ldb_n, M, N, K, nullptr, 0, nullptr, 0, nullptr, 0, M, nullptr, C, 0,
                        gs.local_row0, stream, &gs);
+}
+
+extern "C" int64_t kr_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K) {
+    if (M <= 0 || N <= 0 || K <= 0) return 0;
+    const int64_t tiles = ((M + 127) / 128) * ((N + 127) / 128);
+    const int S = split_k_factor(tiles, K);
+    return S > 1 ? split_k_workspace_bytes(M, N, S) : 0;
+}
+
+extern "C" int kr_gemm_reduce_ws_bf16(const void* A, int64_t lda_m, int64_t lda_k, const void* B, int64_t ldb_k,
+                                      int64_t ldb_n, int64_t M, int64_t N, int64_t K, const void* peers,
+                                      int n_peers, int64_t peers_stride, const void* bias, int64_t band_row0,
+                                      int64_t band_rows, void* c_full, void* out, int out_is_fp32,
+                                      int64_t tile_pivot, void* workspace, int64_t workspace_bytes,
+                                      void* stream) {
+    return gemm_reduce(A, lda_m, lda_k, B, ldb_k, ldb_n, M, N, K, peers, n_peers, nullptr, peers_stride, bias,
+                       band_row0, band_rows, c_full, out, out_is_fp32, tile_pivot, stream, nullptr, workspace,
+                       workspace_bytes);
+}
+
+extern "C" int kr_gemm_reduce_ptrs_ws_bf16(const void* A, int64_t lda_m, int64_t lda_k, const void* B,
+                                           int64_t ldb_k, int64_t ldb_n, int64_t M, int64_t N, int64_t K,
+                                           const void* const* peers, int n_peers, const void* bias,
+                                           int64_t band_row0, int64_t band_rows, void* c_full, void* out,
+                                           int out_is_fp32, int64_t tile_pivot, void* workspace,
+                                           int64_t workspace_bytes, void* stream) {
+    static const void* const kNoPeers[1] = {nullptr};
+    return gemm_reduce(A, lda_m, lda_k, B, ldb_k, ldb_n, M, N, K, peers, n_peers,
+                       peers != nullptr ? peers : kNoPeers, 0, bias, band_row0, band_rows, c_full, out,
+                       out_is_fp32, tile_pivot, stream, nullptr, workspace, workspace_bytes);
 }

@@ -30,6 +30,9 @@ struct GemmArgs {
     int local_row0, local_rows;
     uint64_t wait_ticks;        // bound of one tile's wait, in ticks of the 100 MHz constant clock
     int* status;                // set to 1 + block index by a tile whose wait ran out (may be nullptr)
+    // split K loop of the 128x128 kernel (k_splits == 1: off)
+    int k_splits;               // workgroups per tile, each with its share of the k-steps (grid y)
+    int64_t split_out_stride;   // elements between the fp32 outputs of consecutive splits (0: one output)
     int group_n;         // column panels per scheduling group (tile_schedule)
     int peers_on_mfma;   // 256x256 kernel: add whole-band tiles' peers through the matrix cores
 };
@@ -219,7 +222,7 @@ __device__ __forceinline__ void gemm_epilogue_impl(const GemmArgs& g, const int 
     };
     auto store_out = [&](int64_t off, const float (&f)[8]) __attribute__((always_inline)) {
         if constexpr (F32) {
-            float* o = (float*)g.out + off;
+            float* o = (float*)g.out + (int64_t)blockIdx.y * g.split_out_stride + off;
             *(f32x4*)o = f32x4{f[0], f[1], f[2], f[3]};
             *(f32x4*)(o + 4) = f32x4{f[4], f[5], f[6], f[7]};
         } else {

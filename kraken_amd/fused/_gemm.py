@@ -49,11 +49,49 @@ def prepare_operands(a: torch.Tensor, b: torch.Tensor) -> tuple[torch.Tensor, to
     return a, b
 
 
+_workspaces: dict[tuple[int, int], torch.Tensor] = {}
+
+
+def workspace(dev: torch.device, nbytes: int) -> torch.Tensor | None:
+    """Scratch for the split K loop, one buffer per (device, stream), grown on demand (a
+    buffer per stream keeps calls on different streams from sharing one)."""
+    if nbytes <= 0:
+        return None
+    key = (dev.index if dev.index is not None else torch.cuda.current_device(),
+           torch.cuda.current_stream(dev).cuda_stream)
+    ws = _workspaces.get(key)
+    if ws is None or ws.numel() < nbytes:
+        ws = torch.empty(max(nbytes, 1 << 20), dtype=torch.uint8, device=dev)
+        _workspaces[key] = ws
+    return ws
+
+
 def launch(name, a, b, M, N, peers, n_peers, peers_stride, bias, band_row0, band_rows, c_full, out, pivot):
     """One call of the GEMM entry point; ``peers`` is a ``[P, rows, N]`` tensor (stacked entry
-    point), a list of P tensors (pointer-table entry point) or ``None``."""
+    point), a list of P tensors (pointer-table entry point) or ``None``.  Shapes with few
+    output tiles get a workspace and go through the ``_ws`` entry points (split K loop)."""
     lib = _lib.load()
     out_fp32 = int(out is not None and out.dtype == torch.float32)
+    ws = workspace(a.device, lib.kr_gemm_workspace_bytes(M, N, a.shape[1])) if a.is_cuda else None
+    if ws is not None:
+        if isinstance(peers, (list, tuple)):
+            dev = _lib.require_device(a, b, *peers, bias, c_full, out)
+            table = (ctypes.c_void_p * max(n_peers, 1))(*[t.data_ptr() for t in peers])
+            rc = lib.kr_gemm_reduce_ptrs_ws_bf16(
+                a.data_ptr(), a.stride(0), a.stride(1), b.data_ptr(), b.stride(0), b.stride(1),
+                M, N, a.shape[1], table, n_peers, _lib.ptr(bias), band_row0, band_rows, _lib.ptr(c_full),
+                _lib.ptr(out), out_fp32, pivot, ws.data_ptr(), ws.numel(), _lib.current_stream(dev),
+            )
+        else:
+            dev = _lib.require_device(a, b, peers, bias, c_full, out)
+            rc = lib.kr_gemm_reduce_ws_bf16(
+                a.data_ptr(), a.stride(0), a.stride(1), b.data_ptr(), b.stride(0), b.stride(1),
+                M, N, a.shape[1], _lib.ptr(peers), n_peers, peers_stride, _lib.ptr(bias), band_row0, band_rows,
+                _lib.ptr(c_full), _lib.ptr(out), out_fp32, pivot, ws.data_ptr(), ws.numel(),
+                _lib.current_stream(dev),
+            )
+        _lib.check(rc, name)
+        return
     if isinstance(peers, (list, tuple)):
         dev = _lib.require_device(a, b, *peers, bias, c_full, out)
         table = (ctypes.c_void_p * max(n_peers, 1))(*[t.data_ptr() for t in peers])

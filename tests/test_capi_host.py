@@ -185,6 +185,20 @@ def test_all_gather_matmul_argument_errors(lib):
     assert g(FAKE + 2, 1, None) == _lib.KR_ERR_ALIGNMENT
 
 
+def test_gemm_workspace_entries(lib):
+    assert lib.kr_gemm_workspace_bytes(0, 128, 128) == 0
+    assert lib.kr_gemm_workspace_bytes(8192, 8192, 8192) == 0
+    need = lib.kr_gemm_workspace_bytes(128, 6656, 4096)
+    assert need >= 2 * 128 * 6656 * 4 and need % (128 * 6656 * 4) == 0   # S fp32 partial products
+    f = lib.kr_gemm_reduce_ws_bf16
+    base = (FAKE, 4096, 1, FAKE, 6656, 1, 128, 6656, 4096, None, 0, 0, None, 0, 128, None, FAKE, 0, 0)
+    assert f(*base, FAKE + 8, need, None) == _lib.KR_ERR_ALIGNMENT     # workspace not 16-byte aligned
+    assert f(FAKE, 4096, 2, *base[3:], FAKE, need, None) == _lib.KR_ERR_LAYOUT
+    g = lib.kr_gemm_reduce_ptrs_ws_bf16
+    assert g(FAKE, 4096, 1, FAKE, 6656, 1, 128, 6656, 4096, None, 2, None, 0, 128, None, FAKE, 0, 0,
+             FAKE, need, None) == _lib.KR_ERR_NULL_POINTER
+
+
 def test_striped_share_numel(lib):
     f = lib.kr_striped_share_numel
     numel, W, block = 8 * 37, 4, 16

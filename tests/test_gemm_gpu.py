@@ -5,7 +5,7 @@ import os
 import pytest
 import torch
 
-from kraken_amd import comm, fused
+from kraken_amd import _lib, comm, fused
 from oracle import oracle as orc
 
 pytestmark = pytest.mark.gpu
@@ -351,6 +351,52 @@ def test_separate_peer_buffers_match_the_stacked_form(dev, tile, P):
     o3 = fused.gemm_reduce_scatter_ce_persistent(a.to(dev), b.to(dev), peers=plist, rank=1, world_size=W)
     o4 = fused.gemm_reduce_scatter_ce_persistent(a.to(dev), b.to(dev), peers=peers.to(dev), rank=1, world_size=W)
     assert torch.equal(o3, o4)
+
+
+@pytest.mark.parametrize("splits", [2, 3, 5, 16])
+@pytest.mark.parametrize("b_t", [False, True])
+def test_split_k_loop(dev, monkeypatch, splits, b_t):
+    """Few output tiles: several workgroups share a tile's K loop, their partial products meet
+    in the workspace.  Parity with the oracle for every epilogue form and the same bits run to
+    run (the parts are summed in a fixed order)."""
+    monkeypatch.setenv("KRAKEN_AMD_GEMM_TILE", "128")
+    monkeypatch.setenv("KRAKEN_AMD_GEMM_SPLITK", str(splits))
+    for (M, N, K) in [(128, 384, 1024), (200, 136, 520), (256, 256, 64 * splits)]:
+        a, b, peers = mk(M, N, K, 3, b_t, seed=splits)
+        bias = orc.randn_bf16((N,), 42, 0.02)
+        want = orc.gemm_all_reduce(a, b, peers, bias)
+        ad, bd, pd, biasd = a.to(dev), b.to(dev), peers.to(dev), bias.to(dev)
+        out = fused.gemm_one_shot_all_reduce_fused(ad, bd, peers=pd, bias=biasd)
+        torch.testing.assert_close(out.cpu(), want, rtol=1e-3, atol=1e-3)
+        for _ in range(3):
+            again = fused.gemm_one_shot_all_reduce_fused(ad, bd, peers=pd, bias=biasd)
+            assert torch.equal(out, again)
+        outb = fused.gemm_one_shot_all_reduce_fused(ad, bd, peers=[p for p in pd], bias=biasd, out_dtype=BF16)
+        torch.testing.assert_close(outb.cpu(), want.to(BF16), **TOL)
+        plain = fused.gemm_one_shot_all_reduce_fused(ad, bd)
+        torch.testing.assert_close(plain.cpu(), orc.gemm_all_reduce(a, b), rtol=1e-3, atol=1e-3)
+    # reduce-scatter: band with peers, other bands to the scratch
+    M, N, K, W = 512, 256, 640, 4
+    a, b, _ = mk(M, N, K, 0, b_t)
+    peers = torch.stack([orc.randn_bf16((M // W, N), 100 + j) for j in range(W - 1)])
+    want, c_want = orc.gemm_reduce_scatter(a, b, peers, 2, W)
+    c_scratch = torch.zeros(M, N, dtype=BF16, device=dev)
+    out = fused.gemm_reduce_scatter(a.to(dev), b.to(dev), peers=peers.to(dev), rank=2, c_scratch=c_scratch)
+    torch.testing.assert_close(out.cpu(), want, **TOL)
+    rows = torch.ones(M, dtype=torch.bool)
+    rows[2 * M // W:3 * M // W] = False
+    torch.testing.assert_close(c_scratch.cpu()[rows], c_want[rows], **TOL)
+
+
+def test_split_k_is_chosen_for_few_rows(dev):
+    """The default heuristic: 128 x 6656 x 4096 (52 tiles) asks for a workspace, 4096 x 4096 does not."""
+    lib = _lib.load()
+    assert lib.kr_gemm_workspace_bytes(128, 6656, 4096) > 0
+    assert lib.kr_gemm_workspace_bytes(4096, 4096, 4096) == 0
+    assert lib.kr_gemm_workspace_bytes(128, 6656, 64) == 0          # one k-step: nothing to split
+    a, b, _ = mk(128, 6656, 4096, 0, True)
+    out = fused.gemm_one_shot_all_reduce_fused(a.to(dev), b.to(dev))
+    torch.testing.assert_close(out.cpu(), orc.gemm_all_reduce(a, b), rtol=1e-3, atol=2e-3)
 
 
 def test_gemm_paths_replay_from_a_graph(dev, monkeypatch):
