@@ -206,9 +206,11 @@ int kr_gemm_reduce_ptrs_bf16(const void* A, int64_t lda_m, int64_t lda_k,
                              int64_t tile_pivot, void* stream);
 
 /*
- * kr_gemm_reduce_bf16 / kr_gemm_reduce_ptrs_bf16 with a workspace, for shapes with few output
- * tiles (few rows: M of a few hundred) whose K loop is then split over S workgroups per tile so
- * that all CUs have work.  Two launches: the S partial products go to the workspace in fp32; a
+ * kr_gemm_reduce_bf16 / kr_gemm_reduce_ptrs_bf16 with a workspace, for shapes whose output tiles
+ * do not fill the CUs: few tiles in all (few rows: M of a few hundred), or a last partial round
+ * of 256x256 tiles that is mostly empty (tile count = 256 r + tail, tail <= 96, K >= 4096).
+ * The K loop of those tiles is split over S workgroups per tile.  Two launches (three for the
+ * tail form: the full rounds run as usual first): the S partial products go to the workspace in fp32; a
  * second kernel sums them in the order 0..S-1 and applies the epilogue (peers, bias, band, c_full)
  * with the adds in the same order and the same rounding as the one-pass kernel.  Results are
  * reproducible run to run and differ from the unsplit result only by the fp32 rounding of the

@@ -69,7 +69,7 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_reduce_kernel(const GemmArgs
     const int wm = wave / WN, wn = wave % WN;
 
     int tile_m, tile_n;
-    tile_schedule(g, tile_m, tile_n);
+    tile_schedule(g, schedule_position(g, blockIdx.x), tile_m, tile_n);
     const int m0 = tile_m * BM, n0 = tile_n * BN;
     const uint16_t* a_tile;   // first row of the tile's A panel (gathered matrix or local shard)
     int64_t lda;
@@ -432,6 +432,33 @@ static int split_k_factor(int64_t tiles, int64_t K) {
     s = std::min<int64_t>(s, kMaxSplits);
     return (int)std::max<int64_t>(s, 1);
 }
+// ---- 256x256 kernel: split of the last partial round ------------------------------------------
+// 256 tiles run at a time (one per CU).  When the tile count leaves a last round that is at most
+// 3/8 full and K is long enough, its tiles get S = 256 / tail workgroups each (at least kMinSplitSteps k-steps per
+// part, at most kMaxTailSplits parts), which turns that round from a whole one into tail/256
+// of one; the price is tail * S partial tiles of 256 KiB written and read once.
+constexpr int kMaxTailSplits = 8;
+static void tail_split_plan(int64_t tiles, int64_t K, int* tail_out, int* splits_out) {
+    *tail_out = 0;
+    *splits_out = 1;
+    int64_t force = -1;
+    if (const char* t = getenv("KRAKEN_AMD_GEMM_TAILSPLIT")) force = atoi(t);   // 0: off, n: n parts (testing)
+    if (force == 0 || tiles <= 256) return;
+    const int64_t tail = tiles % 256;
+    // (measured: 16..64 tail tiles gain 5-25 % from K = 4096 on; 128 tail tiles at K = 2048 lose
+    // 12 %: half a round saved does not pay for two more launches and 64 MiB of parts)
+    if (tail == 0 || tail > 96 || (K < 4096 && force <= 0)) return;
+    int64_t s = std::min<int64_t>(256 / tail, kMaxTailSplits);
+    s = std::min<int64_t>(s, (K / 64) / kMinSplitSteps);
+    if (force > 0) s = std::min<int64_t>(force, K / 64);
+    if (s < 2) return;
+    *tail_out = (int)tail;
+    *splits_out = (int)s;
+}
+static int64_t gemm_dtl_tail_workspace_bytes(int tail_tiles, int splits) {
+    return (int64_t)tail_tiles * splits * (256 * 256 * 4);
+}
+
 // workspace of the two-pass form: S fp32 partial products of the whole [M, N] result
 static int64_t split_k_workspace_bytes(int64_t M, int64_t N, int S) { return (int64_t)S * M * N * 4; }
 
@@ -554,6 +581,16 @@ static int gemm_reduce(const void* A, int64_t lda_m, int64_t lda_k, const void* 
     // workgroups share a tile's K loop and meet in the workspace.
     g.k_splits = 1;
     g.split_out_stride = 0;
+    g.tail_tiles = 0;
+    if (dtl && workspace != nullptr && g.progress == nullptr) {
+        int tail, ts;
+        tail_split_plan((int64_t)g.tiles_m * g.tiles_n, K, &tail, &ts);
+        if (tail > 0 && gemm_dtl_tail_workspace_bytes(tail, ts) <= workspace_bytes) {
+            if (!aligned16(workspace)) return KR_ERR_ALIGNMENT;
+            g.tail_tiles = tail;
+            g.k_splits = ts;
+        }
+    }
     int splits = 1;
     if (!dtl && workspace != nullptr) {
         splits = split_k_factor((int64_t)g.tiles_m * g.tiles_n, K);
@@ -582,7 +619,7 @@ static int gemm_reduce(const void* A, int64_t lda_m, int64_t lda_k, const void* 
                            (hipStream_t)stream, g, (const float*)workspace, splits);
         return (int)hipGetLastError();
     }
-    hipError_t e = dtl ? launch_gemm_dtl(g, b_nt, (hipStream_t)stream)
+    hipError_t e = dtl ? launch_gemm_dtl(g, b_nt, (hipStream_t)stream, workspace)
                        : launch_gemm<128, 128, 2, 2>(g, b_nt, even, (hipStream_t)stream);
     return (int)e;
 }
@@ -636,6 +673,16 @@ extern "C" int kr_all_gather_matmul_bf16(const void* A, int64_t lda_m, const voi
 
 extern "C" int64_t kr_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K) {
     if (M <= 0 || N <= 0 || K <= 0) return 0;
+    // the large-tile kernel (same rule as the launch; strides are not known here)
+    const char* force_tile = getenv("KRAKEN_AMD_GEMM_TILE");
+    bool big = (M / 256) * (N / 256) > 128 && K >= 256;
+    if (force_tile != nullptr && force_tile[0] == '1') big = false;
+    if (force_tile != nullptr && force_tile[0] == '2') big = true;
+    if (big && M % 256 == 0 && N % 256 == 0 && K % 64 == 0 && K >= 64) {
+        int tail, ts;
+        tail_split_plan((M / 256) * (N / 256), K, &tail, &ts);
+        return tail > 0 ? gemm_dtl_tail_workspace_bytes(tail, ts) : 0;
+    }
     const int64_t tiles = ((M + 127) / 128) * ((N + 127) / 128);
     const int S = split_k_factor(tiles, K);
     return S > 1 ? split_k_workspace_bytes(M, N, S) : 0;

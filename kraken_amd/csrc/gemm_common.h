@@ -33,13 +33,17 @@ struct GemmArgs {
     // split K loop of the 128x128 kernel (k_splits == 1: off)
     int k_splits;               // workgroups per tile, each with its share of the k-steps (grid y)
     int64_t split_out_stride;   // elements between the fp32 outputs of consecutive splits (0: one output)
+    // 256x256 kernel, split of the last partial round of tiles (tail_tiles == 0: off): the main
+    // launch runs the first tiles_m*tiles_n - tail_tiles tiles of the schedule, a second launch
+    // the remaining ones with k_splits workgroups per tile, a third sums the parts
+    int tail_tiles;
     int group_n;         // column panels per scheduling group (tile_schedule)
     int peers_on_mfma;   // 256x256 kernel: add whole-band tiles' peers through the matrix cores
 };
 
 // LDS-DMA kernel for shapes the 256x256 tile divides (gemm_dtl.hip)
 bool gemm_dtl_supported(const GemmArgs& g);
-hipError_t launch_gemm_dtl(const GemmArgs& g, bool b_nt, hipStream_t st);
+hipError_t launch_gemm_dtl(const GemmArgs& g, bool b_nt, hipStream_t st, void* workspace);
 
 constexpr int kXcds = 8;
 
@@ -86,20 +90,27 @@ __device__ __forceinline__ int64_t wave_uniform(int64_t v) {
     return (int64_t)(((uint64_t)hi << 32) | lo);
 }
 
-// Map the workgroup id to its tile (tile_m, tile_n).
-__device__ __forceinline__ void tile_schedule(const GemmArgs& g, int& tile_m_out, int& tile_n_out) {
-    // ---- tile schedule -------------------------------------------------------------------
-    // Workgroups are dealt round-robin to the 8 XCDs (each with its own L2), so workgroup ids
-    // are first re-numbered to give every XCD a contiguous range of tiles.  Tiles are then
-    // ordered in groups of g.group_n column panels, M fastest in steps of g.group_n columns: the
-    // ~32 tiles an XCD runs at a time form a (32 / group_n) x group_n block that shares its A and
-    // B panels through the XCD's L2 (a dozen panels for 32 tiles), and every XCD works on all row bands -- the rows of the reduce
-    // band (whose tiles also stream the peers' partial sums) are spread over all XCDs
-    // instead of landing on one.  The M order is rotated by the pivot, so the band's (or the
-    // local shard's) tiles are the first ones of every XCD.
-    int pid = blockIdx.x;
+// Position in the tile order of workgroup `wg` of a launch over the first `count` tiles.
+// Workgroups are dealt round-robin to the 8 XCDs (each with its own L2), so workgroup ids are
+// re-numbered to give every XCD a contiguous range of the order: XCD x owns positions
+// [x * ntiles/8, (x+1) * ntiles/8) and a launch over fewer tiles takes the first count/8 of each
+// range (`first` skips positions an earlier launch has taken).
+__device__ __forceinline__ int schedule_position(const GemmArgs& g, int wg, int first = 0) {
     const int ntiles = g.tiles_m * g.tiles_n;
-    if (ntiles % kXcds == 0) pid = (pid % kXcds) * (ntiles / kXcds) + pid / kXcds;
+    if (ntiles % kXcds != 0 || first % kXcds != 0) return first + wg;
+    return (wg % kXcds) * (ntiles / kXcds) + first / kXcds + wg / kXcds;
+}
+
+// Map a position in the tile order to its tile (tile_m, tile_n).
+__device__ __forceinline__ void tile_schedule(const GemmArgs& g, int pid, int& tile_m_out, int& tile_n_out) {
+    // ---- tile schedule -------------------------------------------------------------------
+    // Tiles are ordered in groups of g.group_n column panels, M fastest in steps of g.group_n
+    // columns: the ~32 tiles an XCD runs at a time form a (32 / group_n) x group_n block that
+    // shares its A and B panels through the XCD's L2 (a dozen panels for 32 tiles), and every
+    // XCD works on all row bands -- the rows of the reduce band (whose tiles also stream the
+    // peers' partial sums) are spread over all XCDs instead of landing on one.  The M order is
+    // rotated by the pivot, so the band's (or the local shard's) tiles are the first ones of
+    // every XCD.
     const int per_group = g.group_n * g.tiles_m;
     const int group = pid / per_group;
     const int first_n = group * g.group_n;

@@ -59,7 +59,9 @@ constexpr int kLgkm0 = 0xc07f;   // s_waitcnt lgkmcnt(0) only
 
 // One workgroup tile.  PEERS_FIRST picks the order of the two accumulation phases (peers'
 // partial sums, k loop) for tiles whose peers are added on the matrix cores.
-template <bool B_NT, bool PEERS_FIRST>
+// SPLIT: the workgroup is one of g.k_splits that share a tile of the last partial round: it
+// runs its share of the k-steps and leaves its accumulators in the workspace (no epilogue).
+template <bool B_NT, bool PEERS_FIRST, bool SPLIT = false>
 __device__ __forceinline__ void gemm_dtl_tile(const GemmArgs& g, unsigned char* smem) {
     // Nothing is outstanding at kernel entry; saying so keeps the compiler's own wait-count
     // bookkeeping from carrying the pending loads and stores of the other copy of this code
@@ -72,14 +74,23 @@ __device__ __forceinline__ void gemm_dtl_tile(const GemmArgs& g, unsigned char* 
     const int wm = wave / WN, wn = wave % WN;
 
     int tile_m, tile_n;
-    tile_schedule(g, tile_m, tile_n);
+    const int first_tile = g.tiles_m * g.tiles_n - g.tail_tiles;     // SPLIT: tiles the main launch took
+    const int split = SPLIT ? (int)(blockIdx.x % (unsigned)g.k_splits) : 0;
+    const int tail_index = SPLIT ? (int)(blockIdx.x / (unsigned)g.k_splits) : 0;
+    tile_schedule(g, SPLIT ? schedule_position(g, tail_index, first_tile) : schedule_position(g, blockIdx.x), tile_m,
+                  tile_n);
     const int m0 = tile_m * BM, n0 = tile_n * BN;
+    // k-steps of this workgroup: all of them, or the split's share
+    const int kt_all = g.K / BKD;
+    const int kt_begin = SPLIT ? (int)((int64_t)kt_all * split / g.k_splits) : 0;
+    const int kt_total = SPLIT ? (int)((int64_t)kt_all * (split + 1) / g.k_splits) - kt_begin : kt_all;
+    const int k_begin = kt_begin * BKD;
     const uint16_t* a_tile;   // first row of the tile's A panel (gathered matrix or local shard)
     int64_t lda;
     gathered_a_tile(g, m0, BM, a_tile, lda);
     // (the choice above is the same for the whole workgroup; the descriptor below wants it in
     // scalar registers)
-    a_tile = (const uint16_t*)wave_uniform((int64_t)a_tile);
+    a_tile = (const uint16_t*)wave_uniform((int64_t)a_tile) + k_begin;
     lda = wave_uniform(lda);
 
     // ---- LDS-DMA addressing ----------------------------------------------------------------
@@ -124,9 +135,8 @@ __device__ __forceinline__ void gemm_dtl_tile(const GemmArgs& g, unsigned char* 
                      : "memory", "m0");
     };
     const i32x4 a_rsrc = make_rsrc(a_tile);
-    const i32x4 bt_rsrc = make_rsrc(g.B + (int64_t)n0 * g.ldb);
+    const i32x4 bt_rsrc = make_rsrc(g.B + (int64_t)n0 * g.ldb + (B_NT ? k_begin : 0));
 
-    const int kt_total = g.K / BKD;
     // one LDS-DMA load of k-step t (clamped: the tail re-requests the last tile into a free stage)
     auto issue_load = [&](int t, uint32_t stage, int q) {
         // past the end nothing new is needed, but the per-step load count must not change (the
@@ -144,7 +154,7 @@ __device__ __forceinline__ void gemm_dtl_tile(const GemmArgs& g, unsigned char* 
                          (int)(((int64_t)8 * ch * g.ldb + k0) * 2));
         } else {
             // re-based on the first k-row of the step: the scalar offset stays small for any K
-            lds_dma_b128(make_rsrc(g.B + (int64_t)k0 * g.ldb + n0), B_BASE + stage * B_ST + ch * 1024, b_voff,
+            lds_dma_b128(make_rsrc(g.B + (int64_t)(k_begin + k0) * g.ldb + n0), B_BASE + stage * B_ST + ch * 1024, b_voff,
                          (int)(((int64_t)2 * ch * g.ldb) * 2));
         }
     };
@@ -200,8 +210,8 @@ __device__ __forceinline__ void gemm_dtl_tile(const GemmArgs& g, unsigned char* 
     // values, the same for all four row blocks.
     const int band_lo = g.band_row0;
     const bool tile_in_band = m0 >= band_lo && m0 + BM <= band_lo + g.band_rows;
-    const bool mfma_peers = g.peers_on_mfma && g.n_peers > 0 && tile_in_band;
-    const bool bias_in_acc = g.bias != nullptr && tile_in_band && (g.n_peers == 0 || mfma_peers);
+    const bool mfma_peers = !SPLIT && g.peers_on_mfma && g.n_peers > 0 && tile_in_band;
+    const bool bias_in_acc = !SPLIT && g.bias != nullptr && tile_in_band && (g.n_peers == 0 || mfma_peers);
     f32x16 acc[TM][TN];
     {
         f32x16 init[TN];
@@ -403,6 +413,21 @@ __device__ __forceinline__ void gemm_dtl_tile(const GemmArgs& g, unsigned char* 
     __syncthreads();
 
     pin_accumulators();
+    if constexpr (SPLIT) {
+        // accumulators to the workspace in register order: quad q = (i, j, v/4) of thread tid at
+        // [tail tile][split][q][tid], so that a wave's store is 1 KiB of consecutive addresses
+        f32x4* part = (f32x4*)g.out + ((int64_t)tail_index * g.k_splits + split) * (TM * TN * 4 * WM * WN * 64) + tid;
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+            for (int j = 0; j < TN; ++j)
+#pragma unroll
+                for (int v = 0; v < 4; ++v)
+                    __builtin_nontemporal_store(f32x4{acc[i][j][4 * v], acc[i][j][4 * v + 1], acc[i][j][4 * v + 2],
+                                                      acc[i][j][4 * v + 3]},
+                                                part + ((i * TN + j) * 4 + v) * (WM * WN * 64));
+        return;
+    }
     if (!PEERS_FIRST && mfma_peers) peer_phase();
     pin_accumulators();
     // peers and bias that are already in the accumulators are not added again
@@ -423,13 +448,61 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_dtl_kernel(const GemmArgs g)
 
 }  // namespace
 
+// Second launch of a call with a split tail: g.k_splits workgroups per tile of the last partial
+// round (g.out = workspace).
+template <bool B_NT>
+__global__ __launch_bounds__(WM* WN * 64) void gemm_dtl_split_kernel(const GemmArgs g) {
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+    gemm_dtl_tile<B_NT, false, true>(g, smem);
+}
+
+// Third launch: sums the parts of every tail tile in the order 0..S-1 and applies the epilogue
+// of the one-pass kernel to it (own product in fp32 + peers 0, 1, ... + bias, one rounding).
+// One thread per accumulator quad: block b = (tail tile, quad q), thread tid as in the GEMM
+// kernel; the quad is row wm*128 + 32i + lane%32, columns wn*128 + 32j + 8(v/4) + 4(lane/32) .. +3.
+__global__ __launch_bounds__(WM* WN * 64) void gemm_dtl_tail_finish_kernel(const GemmArgs g, const f32x4* __restrict__ parts) {
+    constexpr int T = WM * WN * 64, NQ = TM * TN * 4;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int u = blockIdx.x / NQ, q = blockIdx.x % NQ;
+    const int S = g.k_splits;
+    const f32x4* p = parts + ((int64_t)u * S * NQ + q) * T + tid;
+    f32x4 sum = {0.0f, 0.0f, 0.0f, 0.0f};
+    for (int sp = 0; sp < S; ++sp) {
+        const f32x4 x = __builtin_nontemporal_load(p + (int64_t)sp * NQ * T);
+        sum.x += x.x; sum.y += x.y; sum.z += x.z; sum.w += x.w;
+    }
+    int tile_m, tile_n;
+    tile_schedule(g, schedule_position(g, u, g.tiles_m * g.tiles_n - g.tail_tiles), tile_m, tile_n);
+    const int i = q / (TN * 4), j = (q / 4) % TN, v4 = q % 4;
+    const int m = tile_m * BM + (wave / WN) * WTM + i * 32 + (lane & 31);
+    const int n = tile_n * BN + (wave % WN) * WTN + j * 32 + 8 * v4 + 4 * (lane >> 5);
+    typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+    const int mb = m - g.band_row0;
+    if (mb < 0 || mb >= g.band_rows) {
+        if (g.c_full != nullptr)
+            *(u32x2*)(g.c_full + (int64_t)m * g.N + n) = u32x2{pack_bf16(sum.x, sum.y), pack_bf16(sum.z, sum.w)};
+        return;
+    }
+    const int64_t off = (int64_t)mb * g.N + n;
+    for (int pq = 0; pq < g.n_peers; ++pq) {
+        const u32x2 w = *(const u32x2*)((const uint16_t*)g.peer.p[pq] + off);
+        sum.x += bf16_lo(w.x); sum.y += bf16_hi(w.x); sum.z += bf16_lo(w.y); sum.w += bf16_hi(w.y);
+    }
+    if (g.bias != nullptr) {
+        const u32x2 w = *(const u32x2*)(g.bias + n);
+        sum.x += bf16_lo(w.x); sum.y += bf16_hi(w.x); sum.z += bf16_lo(w.y); sum.w += bf16_hi(w.y);
+    }
+    if (g.out_is_fp32) *(f32x4*)((float*)g.out + off) = sum;
+    else *(u32x2*)((uint16_t*)g.out + off) = u32x2{pack_bf16(sum.x, sum.y), pack_bf16(sum.z, sum.w)};
+}
+
 bool gemm_dtl_supported(const GemmArgs& g) {
     return g.M % BM == 0 && g.N % BN == 0 && g.K % BKD == 0 && g.K >= BKD &&
            (int64_t)BM * g.lda * 2 < 0x7fffffffLL && (int64_t)(BN > 64 ? BN : 64) * g.ldb * 2 < 0x7fffffffLL;
 }
 
-hipError_t launch_gemm_dtl(const GemmArgs& g, bool b_nt, hipStream_t st) {
-    const dim3 grid((unsigned)(g.tiles_m * g.tiles_n)), block(WM * WN * 64);
+hipError_t launch_gemm_dtl(const GemmArgs& g, bool b_nt, hipStream_t st, void* workspace) {
+    const dim3 grid((unsigned)(g.tiles_m * g.tiles_n - g.tail_tiles)), block(WM * WN * 64);
     static bool opt_in[2] = {false, false};   // benign race: the attribute call is idempotent
     if (!opt_in[b_nt]) {
         hipError_t e = b_nt ? hipFuncSetAttribute((const void*)gemm_dtl_kernel<true>,
@@ -443,6 +516,32 @@ hipError_t launch_gemm_dtl(const GemmArgs& g, bool b_nt, hipStream_t st) {
         hipLaunchKernelGGL(gemm_dtl_kernel<true>, grid, block, LDS_BYTES, st, g);
     else
         hipLaunchKernelGGL(gemm_dtl_kernel<false>, grid, block, LDS_BYTES, st, g);
+    if (g.tail_tiles > 0) {
+        // the tiles of the last partial round: k_splits workgroups each, parts to the workspace,
+        // then the sum and the epilogue
+        static bool split_opt_in[2] = {false, false};
+        if (!split_opt_in[b_nt]) {
+            hipError_t e = b_nt ? hipFuncSetAttribute((const void*)gemm_dtl_split_kernel<true>,
+                                                      hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES)
+                                : hipFuncSetAttribute((const void*)gemm_dtl_split_kernel<false>,
+                                                      hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES);
+            if (e != hipSuccess) return e;
+            split_opt_in[b_nt] = true;
+        }
+        hipError_t e = hipGetLastError();
+        if (e != hipSuccess) return e;
+        GemmArgs gs = g;
+        gs.out = workspace;
+        const dim3 sgrid((unsigned)(g.tail_tiles * g.k_splits));
+        if (b_nt)
+            hipLaunchKernelGGL(gemm_dtl_split_kernel<true>, sgrid, block, LDS_BYTES, st, gs);
+        else
+            hipLaunchKernelGGL(gemm_dtl_split_kernel<false>, sgrid, block, LDS_BYTES, st, gs);
+        e = hipGetLastError();
+        if (e != hipSuccess) return e;
+        hipLaunchKernelGGL(gemm_dtl_tail_finish_kernel, dim3((unsigned)(g.tail_tiles * TM * TN * 4)), block, 0, st, g,
+                           (const f32x4*)workspace);
+    }
     return hipGetLastError();
 }
 

@@ -388,6 +388,45 @@ def test_split_k_loop(dev, monkeypatch, splits, b_t):
     torch.testing.assert_close(c_scratch.cpu()[rows], c_want[rows], **TOL)
 
 
+@pytest.mark.parametrize("b_t", [False, True])
+@pytest.mark.parametrize("force", ["", "3"])
+def test_tail_round_split(dev, monkeypatch, b_t, force):
+    """272 tiles of 256 x 256 = one full round of 256 + 16: the 16 get several workgroups each
+    (second launch) and a finishing pass; every epilogue form against the oracle, and the plain
+    product against the one-launch result."""
+    if force:
+        monkeypatch.setenv("KRAKEN_AMD_GEMM_TAILSPLIT", force)
+    M, N, K, W = 4352, 4096, 4096 if not force else 1024, 2
+    assert _lib.load().kr_gemm_workspace_bytes(M, N, K) == 16 * (int(force) if force else 8) * 256 * 256 * 4
+    a, b, _ = mk(M, N, K, 0, b_t, seed=5)
+    ad, bd = a.to(dev), b.to(dev)
+    prod = a.float() @ b.float()
+    plain = fused.gemm_one_shot_all_reduce_fused(ad, bd)
+    torch.testing.assert_close(plain.cpu(), prod, rtol=1e-3, atol=1e-3)
+    assert torch.equal(plain, fused.gemm_one_shot_all_reduce_fused(ad, bd))          # reproducible
+    monkeypatch.setenv("KRAKEN_AMD_GEMM_TAILSPLIT", "0")
+    one_launch = fused.gemm_one_shot_all_reduce_fused(ad, bd)
+    monkeypatch.setenv("KRAKEN_AMD_GEMM_TAILSPLIT", force) if force else monkeypatch.delenv("KRAKEN_AMD_GEMM_TAILSPLIT")
+    torch.testing.assert_close(plain, one_launch, rtol=1e-4, atol=1e-4)
+    assert not torch.equal(plain, one_launch) or K <= 64                              # the split did run
+    # all-reduce form: peers and bias on every row, bf16 result
+    peers = torch.stack([orc.randn_bf16((M, N), 100 + j) for j in range(2)])
+    bias = orc.randn_bf16((N,), 9, 0.02)
+    out = fused.gemm_one_shot_all_reduce_fused(ad, bd, peers=peers.to(dev), bias=bias.to(dev), out_dtype=BF16)
+    want = (prod + peers.float().sum(0) + bias.float()).to(BF16)
+    torch.testing.assert_close(out.cpu(), want, **TOL)
+    # reduce-scatter form: band of rank 1 (rows 2176.., it starts inside a tile), other rows to the scratch
+    rank = 1
+    bp = torch.stack([orc.randn_bf16((M // W, N), 200 + j) for j in range(W - 1)])
+    c_scratch = torch.zeros(M, N, dtype=BF16, device=dev)
+    out = fused.gemm_reduce_scatter(ad, bd, peers=[p.to(dev) for p in bp], rank=rank, world_size=W, c_scratch=c_scratch)
+    band = slice(rank * (M // W), (rank + 1) * (M // W))
+    torch.testing.assert_close(out.cpu(), (prod[band] + bp.float().sum(0)).to(BF16), **TOL)
+    rows = torch.ones(M, dtype=torch.bool)
+    rows[band] = False
+    torch.testing.assert_close(c_scratch.cpu()[rows], prod[rows].to(BF16), **TOL)
+
+
 def test_split_k_is_chosen_for_few_rows(dev):
     """The default heuristic: 128 x 6656 x 4096 (52 tiles) asks for a workspace, 4096 x 4096 does not."""
     lib = _lib.load()
