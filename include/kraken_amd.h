@@ -140,8 +140,8 @@ int kr_rmsnorm_bf16(const void* x, const void* w, float eps, int64_t rows, int64
  * Rounding: the sum is formed in fp32 and rounded once at the store; with a
  * bf16 result, tiles whose peers are added in the epilogue round the product
  * to bf16 before the sum, as gemm_reduce_scatter_fused.py:72 does.
- * Non-finite input: for shapes the 256x256 kernel takes (M % 256 == N % 256
- * == 0, K % 32 == 0) the peers of tiles lying wholly in the band are added
+ * Non-finite input: for shapes the 256x256 kernel takes (more than 128 tiles
+ * of 256x256, K % 64 == 0) the peers of tiles lying wholly in the band are added
  * on the matrix cores, where an Inf/NaN in a peer also turns the rest of
  * the aligned 32-column block of its row into NaN; KRAKEN_AMD_GEMM_PEERS=epilogue
  * in the environment keeps such values in their own element.

@@ -547,7 +547,7 @@ static int gemm_reduce(const void* A, int64_t lda_m, int64_t lda_k, const void* 
     // tile's epilogue overlaps the other's MFMAs; they also win while all of them fit on the
     // 256 CUs at once (512 tiles = 128 of the large ones): measured, the large tile is 15-30 %
     // faster from 144 tiles on and 5-10 % slower at 128, for K from 1024 to 8192.
-    bool big = (M / 256) * (N / 256) > 128 && K >= 256;
+    bool big = ((M + 255) / 256) * ((N + 255) / 256) > 128 && K >= 256;
     // KRAKEN_AMD_GEMM_TILE=128|256 overrides the choice (testing and tuning)
     if (const char* t = getenv("KRAKEN_AMD_GEMM_TILE")) {
         if (t[0] == '1') big = false;
@@ -582,7 +582,7 @@ static int gemm_reduce(const void* A, int64_t lda_m, int64_t lda_k, const void* 
     g.k_splits = 1;
     g.split_out_stride = 0;
     g.tail_tiles = 0;
-    if (dtl && workspace != nullptr && g.progress == nullptr) {
+    if (dtl && workspace != nullptr && g.progress == nullptr && M % 256 == 0 && N % 256 == 0) {
         int tail, ts;
         tail_split_plan((int64_t)g.tiles_m * g.tiles_n, K, &tail, &ts);
         if (tail > 0 && gemm_dtl_tail_workspace_bytes(tail, ts) <= workspace_bytes) {
@@ -675,10 +675,11 @@ extern "C" int64_t kr_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K) {
     if (M <= 0 || N <= 0 || K <= 0) return 0;
     // the large-tile kernel (same rule as the launch; strides are not known here)
     const char* force_tile = getenv("KRAKEN_AMD_GEMM_TILE");
-    bool big = (M / 256) * (N / 256) > 128 && K >= 256;
+    bool big = ((M + 255) / 256) * ((N + 255) / 256) > 128 && K >= 256;
     if (force_tile != nullptr && force_tile[0] == '1') big = false;
     if (force_tile != nullptr && force_tile[0] == '2') big = true;
-    if (big && M % 256 == 0 && N % 256 == 0 && K % 64 == 0 && K >= 64) {
+    if (big && K % 64 == 0 && K >= 64) {
+        if (M % 256 != 0 || N % 256 != 0) return 0;
         int tail, ts;
         tail_split_plan((M / 256) * (N / 256), K, &tail, &ts);
         return tail > 0 ? gemm_dtl_tail_workspace_bytes(tail, ts) : 0;

@@ -1,5 +1,5 @@
-// bf16 GEMM main loop with direct global->LDS loads ("LDS DMA") for shapes the 256x256 tile
-// divides:  M % 256 == 0, N % 256 == 0, K % 64 == 0.
+// bf16 GEMM main loop with direct global->LDS loads ("LDS DMA"), 256x256 tiles, for K % 64 == 0
+// (M and N may be ragged: the tiles at the lower and right edge are handled below).
 //
 // Workgroup tile 256 x 256, four wavefronts (2 x 2), each owning 128 x 128 of C as 4 x 4
 // v_mfma_f32_32x32x16_bf16 accumulators (256 AGPRs).  The k loop advances 64 at a time through a
@@ -61,7 +61,8 @@ constexpr int kLgkm0 = 0xc07f;   // s_waitcnt lgkmcnt(0) only
 // partial sums, k loop) for tiles whose peers are added on the matrix cores.
 // SPLIT: the workgroup is one of g.k_splits that share a tile of the last partial round: it
 // runs its share of the k-steps and leaves its accumulators in the workspace (no epilogue).
-template <bool B_NT, bool PEERS_FIRST, bool SPLIT = false>
+// RAGGED: M or N is not a multiple of 256 (edge tiles get the bounds-checked epilogue).
+template <bool B_NT, bool PEERS_FIRST, bool SPLIT = false, bool RAGGED = false>
 __device__ __forceinline__ void gemm_dtl_tile(const GemmArgs& g, unsigned char* smem) {
     // Nothing is outstanding at kernel entry; saying so keeps the compiler's own wait-count
     // bookkeeping from carrying the pending loads and stores of the other copy of this code
@@ -112,10 +113,16 @@ __device__ __forceinline__ void gemm_dtl_tile(const GemmArgs& g, unsigned char* 
     }
     // Buffer resource descriptor: 48-bit base, stride 0 (raw), 2^31-1 bytes, 32-bit data format.
     typedef int i32x4 __attribute__((ext_vector_type(4)));
-    auto make_rsrc = [](const void* base) {
+    auto make_rsrc = [](const void* base, int64_t bytes = 0x7fffffff) {
         const uint64_t b = (uint64_t)base;
-        return i32x4{(int)(uint32_t)b, (int)(uint32_t)((b >> 32) & 0xffff), 0x7fffffff, 0x00020000};
+        return i32x4{(int)(uint32_t)b, (int)(uint32_t)((b >> 32) & 0xffff),
+                     (int)(bytes < 0x7fffffff ? (bytes > 0 ? bytes : 0) : 0x7fffffff), 0x00020000};
     };
+    // A tile at the lower or right edge of a ragged shape has fewer than 256 valid rows (columns):
+    // its operand descriptors end with the last valid row, so the loads of the missing rows are
+    // out of range (they fetch nothing) and the accumulators of those rows and columns, which
+    // hold whatever the LDS stage held, are never stored (the epilogue masks them).
+    const int rows_a = RAGGED ? min(BM, g.M - m0) : BM, rows_b = RAGGED ? min(BN, g.N - n0) : BN;
     // The LDS-DMA load is issued through inline assembly on purpose: the compiler then does not
     // know that LDS is written behind its back and leaves the ordering to the explicit
     // s_waitcnt vmcnt / s_barrier pairs below (told about it, it waits for vmcnt(0) in front of
@@ -134,8 +141,10 @@ __device__ __forceinline__ void gemm_dtl_tile(const GemmArgs& g, unsigned char* 
                      : "s"(lds_addr), "v"(voff), "s"(rsrc), "s"(soff)
                      : "memory", "m0");
     };
-    const i32x4 a_rsrc = make_rsrc(a_tile);
-    const i32x4 bt_rsrc = make_rsrc(g.B + (int64_t)n0 * g.ldb + (B_NT ? k_begin : 0));
+    const i32x4 a_rsrc = RAGGED ? make_rsrc(a_tile, ((int64_t)(rows_a - 1) * lda + (g.K - k_begin)) * 2) : make_rsrc(a_tile);
+    const i32x4 bt_rsrc = RAGGED ? make_rsrc(g.B + (int64_t)n0 * g.ldb + (B_NT ? k_begin : 0),
+                                             ((int64_t)(rows_b - 1) * g.ldb + (g.K - k_begin)) * 2)
+                                 : make_rsrc(g.B + (int64_t)n0 * g.ldb + (B_NT ? k_begin : 0));
 
     // one LDS-DMA load of k-step t (clamped: the tail re-requests the last tile into a free stage)
     auto issue_load = [&](int t, uint32_t stage, int q) {
@@ -154,7 +163,12 @@ __device__ __forceinline__ void gemm_dtl_tile(const GemmArgs& g, unsigned char* 
                          (int)(((int64_t)8 * ch * g.ldb + k0) * 2));
         } else {
             // re-based on the first k-row of the step: the scalar offset stays small for any K
-            lds_dma_b128(make_rsrc(g.B + (int64_t)(k_begin + k0) * g.ldb + n0), B_BASE + stage * B_ST + ch * 1024, b_voff,
+            // (the descriptor ends with the matrix: columns past N of the last k-rows fetch nothing, those of
+            // other k-rows read the next row's first columns -- neither reaches a stored element)
+            lds_dma_b128(RAGGED ? make_rsrc(g.B + (int64_t)(k_begin + k0) * g.ldb + n0,
+                                            ((int64_t)(g.K - 1 - (k_begin + k0)) * g.ldb + (g.N - n0)) * 2)
+                                : make_rsrc(g.B + (int64_t)(k_begin + k0) * g.ldb + n0),
+                         B_BASE + stage * B_ST + ch * 1024, b_voff,
                          (int)(((int64_t)2 * ch * g.ldb) * 2));
         }
     };
@@ -209,7 +223,8 @@ __device__ __forceinline__ void gemm_dtl_tile(const GemmArgs& g, unsigned char* 
     // column 32j + 8(v/4) + 4(lane/32) + v%4, so a lane needs 16 groups of 4 consecutive bias
     // values, the same for all four row blocks.
     const int band_lo = g.band_row0;
-    const bool tile_in_band = m0 >= band_lo && m0 + BM <= band_lo + g.band_rows;
+    const bool full_tile = !RAGGED || (m0 + BM <= g.M && n0 + BN <= g.N);
+    const bool tile_in_band = full_tile && m0 >= band_lo && m0 + BM <= band_lo + g.band_rows;
     const bool mfma_peers = !SPLIT && g.peers_on_mfma && g.n_peers > 0 && tile_in_band;
     const bool bias_in_acc = !SPLIT && g.bias != nullptr && tile_in_band && (g.n_peers == 0 || mfma_peers);
     f32x16 acc[TM][TN];
@@ -431,19 +446,23 @@ __device__ __forceinline__ void gemm_dtl_tile(const GemmArgs& g, unsigned char* 
     if (!PEERS_FIRST && mfma_peers) peer_phase();
     pin_accumulators();
     // peers and bias that are already in the accumulators are not added again
-    gemm_epilogue<BM, WTM, WTN, TM, TN, true, EP_WAVE>(g, mfma_peers ? 0 : g.n_peers, bias_in_acc ? nullptr : g.bias,
-                                                       acc, smem, m0, n0, wm, wn, lane, wave);
+    if (full_tile) {
+        gemm_epilogue<BM, WTM, WTN, TM, TN, true, EP_WAVE>(g, mfma_peers ? 0 : g.n_peers, bias_in_acc ? nullptr : g.bias,
+                                                           acc, smem, m0, n0, wm, wn, lane, wave);
+    } else if constexpr (RAGGED) {   // edge tile: every access checked against M and N
+        gemm_epilogue<BM, WTM, WTN, TM, TN, false, EP_WAVE>(g, g.n_peers, g.bias, acc, smem, m0, n0, wm, wn, lane, wave);
+    }
 }
 #undef KR_SCHED_FENCE
 
 // The two phase orders are two complete copies of the tile code under one uniform branch: each
 // copy is straight-line (phase, phase, epilogue), which keeps the 256 accumulators in their
 // registers; one copy with a run-time order has the register allocator move them through memory.
-template <bool B_NT>
+template <bool B_NT, bool RAGGED>
 __global__ __launch_bounds__(WM* WN * 64) void gemm_dtl_kernel(const GemmArgs g) {
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];   // starts at LDS address 0
-    if (g.peers_on_mfma && g.n_peers > 0 && (g.peers_on_mfma == 1 ? ((blockIdx.x >> 3) & 1) : g.peers_on_mfma == 2)) gemm_dtl_tile<B_NT, true>(g, smem);
-    else gemm_dtl_tile<B_NT, false>(g, smem);
+    if (g.peers_on_mfma && g.n_peers > 0 && (g.peers_on_mfma == 1 ? ((blockIdx.x >> 3) & 1) : g.peers_on_mfma == 2)) gemm_dtl_tile<B_NT, true, false, RAGGED>(g, smem);
+    else gemm_dtl_tile<B_NT, false, false, RAGGED>(g, smem);
 }
 
 }  // namespace
@@ -497,25 +516,29 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_dtl_tail_finish_kernel(const
 }
 
 bool gemm_dtl_supported(const GemmArgs& g) {
-    return g.M % BM == 0 && g.N % BN == 0 && g.K % BKD == 0 && g.K >= BKD &&
+    return g.K % BKD == 0 && g.K >= BKD &&
            (int64_t)BM * g.lda * 2 < 0x7fffffffLL && (int64_t)(BN > 64 ? BN : 64) * g.ldb * 2 < 0x7fffffffLL;
 }
 
 hipError_t launch_gemm_dtl(const GemmArgs& g, bool b_nt, hipStream_t st, void* workspace) {
     const dim3 grid((unsigned)(g.tiles_m * g.tiles_n - g.tail_tiles)), block(WM * WN * 64);
-    static bool opt_in[2] = {false, false};   // benign race: the attribute call is idempotent
-    if (!opt_in[b_nt]) {
-        hipError_t e = b_nt ? hipFuncSetAttribute((const void*)gemm_dtl_kernel<true>,
-                                                  hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES)
-                            : hipFuncSetAttribute((const void*)gemm_dtl_kernel<false>,
-                                                  hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES);
+    const bool ragged = g.M % BM != 0 || g.N % BN != 0;
+    const void* kfn = b_nt ? (ragged ? (const void*)gemm_dtl_kernel<true, true> : (const void*)gemm_dtl_kernel<true, false>)
+                           : (ragged ? (const void*)gemm_dtl_kernel<false, true> : (const void*)gemm_dtl_kernel<false, false>);
+    static bool opt_in[4] = {false, false, false, false};   // benign race: the attribute call is idempotent
+    const int which = (b_nt ? 2 : 0) + (ragged ? 1 : 0);
+    if (!opt_in[which]) {
+        hipError_t e = hipFuncSetAttribute(kfn, hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES);
         if (e != hipSuccess) return e;
-        opt_in[b_nt] = true;
+        opt_in[which] = true;
     }
-    if (b_nt)
-        hipLaunchKernelGGL(gemm_dtl_kernel<true>, grid, block, LDS_BYTES, st, g);
-    else
-        hipLaunchKernelGGL(gemm_dtl_kernel<false>, grid, block, LDS_BYTES, st, g);
+    if (b_nt) {
+        if (ragged) hipLaunchKernelGGL((gemm_dtl_kernel<true, true>), grid, block, LDS_BYTES, st, g);
+        else hipLaunchKernelGGL((gemm_dtl_kernel<true, false>), grid, block, LDS_BYTES, st, g);
+    } else {
+        if (ragged) hipLaunchKernelGGL((gemm_dtl_kernel<false, true>), grid, block, LDS_BYTES, st, g);
+        else hipLaunchKernelGGL((gemm_dtl_kernel<false, false>), grid, block, LDS_BYTES, st, g);
+    }
     if (g.tail_tiles > 0) {
         // the tiles of the last partial round: k_splits workgroups each, parts to the workspace,
         // then the sum and the epilogue

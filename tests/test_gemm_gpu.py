@@ -427,6 +427,37 @@ def test_tail_round_split(dev, monkeypatch, b_t, force):
     torch.testing.assert_close(c_scratch.cpu()[rows], prod[rows].to(BF16), **TOL)
 
 
+@pytest.mark.parametrize("b_t", [False, True])
+def test_ragged_shapes_on_the_large_tile(dev, monkeypatch, b_t):
+    """M and N that 256 does not divide, on the 256 x 256 kernel: edge tiles read short operand
+    panels and store through the bounds-checked epilogue; every epilogue form."""
+    monkeypatch.setenv("KRAKEN_AMD_GEMM_TILE", "256")
+    for (M, N, K) in [(1000, 520, 192), (300, 264, 64), (513, 1032, 256), (768, 8, 128), (8, 768, 128)]:
+        a, b, peers = mk(M, N, K, 2, b_t, seed=M)
+        bias = orc.randn_bf16((N,), 42, 0.02)
+        ad, bd, pd, biasd = a.to(dev), b.to(dev), peers.to(dev), bias.to(dev)
+        want = orc.gemm_all_reduce(a, b, peers, bias)
+        out = fused.gemm_one_shot_all_reduce_fused(ad, bd, peers=pd, bias=biasd)
+        torch.testing.assert_close(out.cpu(), want, rtol=1e-3, atol=1e-3)
+        outb = fused.gemm_one_shot_all_reduce_fused(ad, bd, peers=pd, bias=biasd, out_dtype=BF16)
+        torch.testing.assert_close(outb.cpu(), want.to(BF16), **TOL)
+        plain = fused.gemm_one_shot_all_reduce_fused(ad, bd, out_dtype=BF16)
+        torch.testing.assert_close(plain.cpu(), orc.gemm_all_reduce(a, b).to(BF16), **TOL)
+    # reduce-scatter with a band that ends inside the ragged last tile; guard rows behind the outputs
+    M, N, K, W = 1000, 520, 192, 4
+    a, b, _ = mk(M, N, K, 0, b_t, seed=3)
+    for rank in (0, 3):
+        bp = torch.stack([orc.randn_bf16((M // W, N), 300 + j) for j in range(W - 1)])
+        want, c_want = orc.gemm_reduce_scatter(a, b, bp, rank, W)
+        c_scratch = torch.zeros(M + 8, N, dtype=BF16, device=dev)
+        out = fused.gemm_reduce_scatter(a.to(dev), b.to(dev), peers=bp.to(dev), rank=rank, c_scratch=c_scratch[:M])
+        torch.testing.assert_close(out.cpu(), want, **TOL)
+        rows = torch.ones(M, dtype=torch.bool)
+        rows[rank * (M // W):(rank + 1) * (M // W)] = False
+        torch.testing.assert_close(c_scratch.cpu()[:M][rows], c_want[rows], **TOL)
+        assert (c_scratch[M:] == 0).all()                     # nothing written past row M
+
+
 def test_split_k_is_chosen_for_few_rows(dev):
     """The default heuristic: 128 x 6656 x 4096 (52 tiles) asks for a workspace, 4096 x 4096 does not."""
     lib = _lib.load()
