@@ -17,8 +17,13 @@ enum RowBias { kRowNoBias = 0, kRowFullBias = 1, kRowVecBias = 2 };
 
 constexpr int kMaxVpt = 8;       // vectors per thread  -> D <= 1024 * 8 * 8
 constexpr int kMaxThreads = 1024;
+constexpr int64_t kLatRows = 1024;  // at most this many rows: latency-first kernel
 
-template <class SRC, int VPT, int WT, int BIAS>
+// LAT (few rows: the kernel's time is one workgroup's latency): every load of the thread --
+// weights, bias, the W inputs -- is issued before the first is consumed and none sits under a
+// branch (a lane past the end of the row re-reads the row's last vector and is masked), so the
+// row costs one memory round trip instead of three.
+template <class SRC, int VPT, int WT, int BIAS, bool LAT = false>
 __global__ __launch_bounds__(kMaxThreads) void reduce_rmsnorm_kernel(
     const SRC src, int w_rt, int d_vec,
     const u32x4* __restrict__ bias, const u32x4* __restrict__ wgt, float eps, float inv_d,
@@ -36,6 +41,32 @@ __global__ __launch_bounds__(kMaxThreads) void reduce_rmsnorm_kernel(
     // enough to need 4+ vectors per thread fetch them after the reduction instead, to stay
     // inside the 128 registers a 1024-thread workgroup leaves per thread
     constexpr bool kEarlyWeights = VPT < 4;
+    constexpr bool kLatPath = LAT && WT > 0 && WT * VPT <= 16 && VPT == 1;
+    if constexpr (kLatPath) {
+        u32x4 bv[VPT];
+        u32x4 x[WT][VPT];
+#pragma unroll
+        for (int v = 0; v < VPT; ++v) {
+            const int cc = min(tid + v * nthr, d_vec - 1);
+            wv[v] = wgt[cc];
+            if (BIAS == kRowFullBias) bv[v] = ld_stream(bias + row_v + cc);
+            else if (BIAS == kRowVecBias) bv[v] = bias[cc];
+        }
+#pragma unroll
+        for (int r = 0; r < WT; ++r)
+#pragma unroll
+            for (int v = 0; v < VPT; ++v) x[r][v] = ld_stream(src.at(r) + row_v + min(tid + v * nthr, d_vec - 1));
+#pragma unroll
+        for (int v = 0; v < VPT; ++v) {
+            if (BIAS == kRowNoBias) zero8(s[v]);
+            else unpack8(bv[v], s[v]);
+#pragma unroll
+            for (int r = 0; r < WT; ++r) add8(x[r][v], s[v]);
+            const bool live = tid + v * nthr < d_vec;
+#pragma unroll
+            for (int j = 0; j < 8; ++j) s[v][j] = live ? s[v][j] : 0.0f;
+        }
+    } else {
     if (kEarlyWeights) {
 #pragma unroll
         for (int v = 0; v < VPT; ++v) {
@@ -92,6 +123,8 @@ __global__ __launch_bounds__(kMaxThreads) void reduce_rmsnorm_kernel(
         }
     }
 
+    }   // !kLatPath
+
     float ss = 0.0f;
 #pragma unroll
     for (int v = 0; v < VPT; ++v)
@@ -122,37 +155,37 @@ __global__ __launch_bounds__(kMaxThreads) void reduce_rmsnorm_kernel(
     }
 }
 
-template <class SRC, int VPT, int WT>
+template <class SRC, int VPT, int WT, bool LAT>
 static hipError_t launch_row2(int mode, dim3 grid, dim3 block, hipStream_t st, const SRC& tab, int W,
                               int d_vec, const u32x4* bias, const u32x4* wgt, float eps,
                               float inv_d, u32x4* y) {
     switch (mode) {
         case kRowNoBias:
-            hipLaunchKernelGGL((reduce_rmsnorm_kernel<SRC, VPT, WT, kRowNoBias>), grid, block, 0, st, tab, W,
+            hipLaunchKernelGGL((reduce_rmsnorm_kernel<SRC, VPT, WT, kRowNoBias, LAT>), grid, block, 0, st, tab, W,
                                d_vec, bias, wgt, eps, inv_d, y);
             break;
         case kRowFullBias:
-            hipLaunchKernelGGL((reduce_rmsnorm_kernel<SRC, VPT, WT, kRowFullBias>), grid, block, 0, st, tab, W,
+            hipLaunchKernelGGL((reduce_rmsnorm_kernel<SRC, VPT, WT, kRowFullBias, LAT>), grid, block, 0, st, tab, W,
                                d_vec, bias, wgt, eps, inv_d, y);
             break;
         default:
-            hipLaunchKernelGGL((reduce_rmsnorm_kernel<SRC, VPT, WT, kRowVecBias>), grid, block, 0, st, tab, W,
+            hipLaunchKernelGGL((reduce_rmsnorm_kernel<SRC, VPT, WT, kRowVecBias, LAT>), grid, block, 0, st, tab, W,
                                d_vec, bias, wgt, eps, inv_d, y);
             break;
     }
     return hipGetLastError();
 }
 
-template <class SRC, int VPT>
+template <class SRC, int VPT, bool LAT>
 static hipError_t launch_row1(int W, int mode, dim3 grid, dim3 block, hipStream_t st, const SRC& tab,
                               int d_vec, const u32x4* bias, const u32x4* wgt, float eps,
                               float inv_d, u32x4* y) {
     switch (W) {
-        case 1: return launch_row2<SRC, VPT, 1>(mode, grid, block, st, tab, W, d_vec, bias, wgt, eps, inv_d, y);
-        case 2: return launch_row2<SRC, VPT, 2>(mode, grid, block, st, tab, W, d_vec, bias, wgt, eps, inv_d, y);
-        case 4: return launch_row2<SRC, VPT, 4>(mode, grid, block, st, tab, W, d_vec, bias, wgt, eps, inv_d, y);
-        case 8: return launch_row2<SRC, VPT, 8>(mode, grid, block, st, tab, W, d_vec, bias, wgt, eps, inv_d, y);
-        default: return launch_row2<SRC, VPT, 0>(mode, grid, block, st, tab, W, d_vec, bias, wgt, eps, inv_d, y);
+        case 1: return launch_row2<SRC, VPT, 1, LAT>(mode, grid, block, st, tab, W, d_vec, bias, wgt, eps, inv_d, y);
+        case 2: return launch_row2<SRC, VPT, 2, LAT>(mode, grid, block, st, tab, W, d_vec, bias, wgt, eps, inv_d, y);
+        case 4: return launch_row2<SRC, VPT, 4, LAT>(mode, grid, block, st, tab, W, d_vec, bias, wgt, eps, inv_d, y);
+        case 8: return launch_row2<SRC, VPT, 8, LAT>(mode, grid, block, st, tab, W, d_vec, bias, wgt, eps, inv_d, y);
+        default: return launch_row2<SRC, VPT, 0, LAT>(mode, grid, block, st, tab, W, d_vec, bias, wgt, eps, inv_d, y);
     }
 }
 
@@ -181,6 +214,11 @@ static int launch_rows(const SRC& tab, int W, int64_t rows, int64_t D, const voi
     int threads, vpt;
     const int d_vec = (int)(D / 8);
     row_geometry(d_vec, &threads, &vpt);
+    // few rows of at most 8192 elements: one workgroup's latency is the kernel's time, and the
+    // latency-first instantiation is 9 % faster at [256, 4096], 2.5 % at [16, 8192]; with many
+    // rows it is level or up to 2 % slower (KRAKEN_AMD_ROW_LAT=0|1 overrides, for tuning)
+    bool lat = rows <= kLatRows;
+    if (const char* e = getenv("KRAKEN_AMD_ROW_LAT")) lat = e[0] == '1';
     const dim3 grid((unsigned)rows), block((unsigned)threads);
     const hipStream_t st = (hipStream_t)stream;
     const u32x4* bp = (const u32x4*)bias;
@@ -189,10 +227,13 @@ static int launch_rows(const SRC& tab, int W, int64_t rows, int64_t D, const voi
     const float inv_d = 1.0f / (float)D;
     hipError_t e;
     switch (vpt) {
-        case 1: e = launch_row1<SRC, 1>(W, mode, grid, block, st, tab, d_vec, bp, wp, eps, inv_d, yp); break;
-        case 2: e = launch_row1<SRC, 2>(W, mode, grid, block, st, tab, d_vec, bp, wp, eps, inv_d, yp); break;
-        case 4: e = launch_row1<SRC, 4>(W, mode, grid, block, st, tab, d_vec, bp, wp, eps, inv_d, yp); break;
-        default: e = launch_row1<SRC, 8>(W, mode, grid, block, st, tab, d_vec, bp, wp, eps, inv_d, yp); break;
+        case 1:
+            e = lat ? launch_row1<SRC, 1, true>(W, mode, grid, block, st, tab, d_vec, bp, wp, eps, inv_d, yp)
+                    : launch_row1<SRC, 1, false>(W, mode, grid, block, st, tab, d_vec, bp, wp, eps, inv_d, yp);
+            break;
+        case 2: e = launch_row1<SRC, 2, false>(W, mode, grid, block, st, tab, d_vec, bp, wp, eps, inv_d, yp); break;
+        case 4: e = launch_row1<SRC, 4, false>(W, mode, grid, block, st, tab, d_vec, bp, wp, eps, inv_d, yp); break;
+        default: e = launch_row1<SRC, 8, false>(W, mode, grid, block, st, tab, d_vec, bp, wp, eps, inv_d, yp); break;
     }
     return (int)e;
 }
