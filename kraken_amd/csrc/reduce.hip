@@ -150,8 +150,14 @@ __global__ __launch_bounds__(kThreads) void reduce_rotated_kernel(
 }
 
 // Vectors per thread per block: 4 for large inputs (most bytes in flight per workgroup), 1
-// for inputs too small to give every CU four such blocks (more, smaller workgroups).
-static int pick_unroll(int64_t nvec) { return nvec >= (int64_t)kMaxBlocks * kThreads * 4 ? 4 : 1; }
+// for inputs too small to give every CU such a block (more, smaller workgroups).  Measured with
+// inputs that are not in any cache: from 256 blocks of 4 x 256 vectors on (one per CU) the
+// larger block wins whenever the blocks fill whole rounds of 256 CUs (32 MiB input: 9.0 -> 7.9 us,
+// 64 MiB: 16.0 -> 13.5 us), and loses 5 % at one and a half rounds.
+static int pick_unroll(int64_t nvec) {
+    const int64_t blocks4 = (nvec + kThreads * 4 - 1) / (kThreads * 4);
+    return (blocks4 >= 768 || (blocks4 >= 256 && blocks4 % 256 == 0)) ? 4 : 1;
+}
 
 template <class SRC, int WT, int BIAS, bool BF>
 static void launch_reduce3(hipStream_t s, const SRC& tab, int W, int64_t nvec, const u32x4* bias,
