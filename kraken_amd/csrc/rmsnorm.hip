@@ -6,7 +6,7 @@
 // W*D*2 B of slices (+ D*2 bias + D*2 weight) in, D*2 B out per row.  The sum
 // of squares is reduced inside each wavefront with DPP lane permutes, then
 // across the wavefronts of the workgroup through a few words of LDS that every
-// thread re-reads in the same order, so all threads hold the same rstd.
+// wavefront re-reads and sums in the same way, so all threads hold the same rstd.
 #include <stdlib.h>
 
 #include "common.h"
@@ -137,8 +137,10 @@ __global__ __launch_bounds__(kMaxThreads) void reduce_rmsnorm_kernel(
     if (nwaves > 1) {
         if ((tid & (kWave - 1)) == 0) wave_part[tid / kWave] = ss;
         __syncthreads();
-        total = 0.0f;
-        for (int i = 0; i < nwaves; ++i) total += wave_part[i];
+        // lane i of every wave fetches wave i's part (one LDS read instead of nwaves in a row)
+        // and the wave sums them the same way: all threads hold the same total
+        const int l = tid & (kWave - 1);
+        total = wave_sum(l < nwaves ? wave_part[l] : 0.0f);
     }
     const float rstd = __builtin_amdgcn_rsqf(total * inv_d + eps);
 
