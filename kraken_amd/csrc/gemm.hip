@@ -542,8 +542,8 @@ static int gemm_reduce(const void* A, int64_t lda_m, int64_t lda_k, const void* 
     g.out_is_fp32 = out_is_fp32;
 
     // Tile choice: the 256x256 tile of the LDS-DMA kernel (4 waves x 128x128) has the highest
-    // MFMA work per LDS/HBM byte; it needs a shape it divides and a K loop long enough to
-    // amortise its epilogue.  Otherwise 128x128 tiles, two of which share a CU so that one
+    // MFMA work per LDS/HBM byte; it needs K % 64 == 0 and a K loop long enough to amortise
+    // its epilogue.  Otherwise 128x128 tiles, two of which share a CU so that one
     // tile's epilogue overlaps the other's MFMAs; they also win while all of them fit on the
     // 256 CUs at once (512 tiles = 128 of the large ones): measured, the large tile is 15-30 %
     // faster from 144 tiles on and 5-10 % slower at 128, for K from 1024 to 8192.
