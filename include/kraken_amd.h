@@ -208,7 +208,8 @@ int kr_gemm_reduce_ptrs_bf16(const void* A, int64_t lda_m, int64_t lda_k,
 /*
  * kr_gemm_reduce_bf16 / kr_gemm_reduce_ptrs_bf16 with a workspace, for shapes whose output tiles
  * do not fill the CUs: few tiles in all (few rows: M of a few hundred), or a last partial round
- * of 256x256 tiles that is mostly empty (tile count = 256 r + tail, tail <= 96, K >= 4096).
+ * of 256x256 tiles that is mostly empty (tile count = 256 r + tail, tail <= 96, K >= 4096; with
+ * r = 0 and a long K loop all tiles are such a tail).
  * The K loop of those tiles is split over S workgroups per tile.  Two launches (three for the
  * tail form: the full rounds run as usual first): the S partial products go to the workspace in fp32; a
  * second kernel sums them in the order 0..S-1 and applies the epilogue (peers, bias, band, c_full)

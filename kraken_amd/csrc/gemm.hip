@@ -426,6 +426,9 @@ static int split_k_factor(int64_t tiles, int64_t K) {
         const int v = atoi(t);
         if (v >= 1 && v <= kMaxSplits) return (int)std::min<int64_t>(v, std::max<int64_t>(1, (K + BK - 1) / BK));
     }
+    // (up to 256 tiles a second workgroup per tile still finds a place next to the first; it pays
+    // once the K loop is long: 208 tiles at K = 16384 measured 197 -> 178 us, at K = 4096 54 -> 62 us)
+    if (tiles > 128 && tiles <= 256 && K >= 12288) return 2;
     if (tiles <= 0 || tiles * 2 > 256) return 1;
     int64_t s = 256 / tiles;
     s = std::min<int64_t>(s, ((K + BK - 1) / BK) / kMinSplitSteps);
@@ -443,11 +446,12 @@ static void tail_split_plan(int64_t tiles, int64_t K, int* tail_out, int* splits
     *splits_out = 1;
     int64_t force = -1;
     if (const char* t = getenv("KRAKEN_AMD_GEMM_TAILSPLIT")) force = atoi(t);   // 0: off, n: n parts (testing)
-    if (force == 0 || tiles <= 256) return;
+    if (force == 0 || (tiles > 128 && tiles <= 256)) return;
+    // up to 128 tiles the whole launch is one partial round
     const int64_t tail = tiles % 256;
     // (measured: 16..64 tail tiles gain 5-25 % from K = 4096 on; 128 tail tiles at K = 2048 lose
     // 12 %: half a round saved does not pay for two more launches and 64 MiB of parts)
-    if (tail == 0 || tail > 96 || (K < 4096 && force <= 0)) return;
+    if (tail == 0 || (tail > 96 && tiles > 128) || (K < 4096 && force <= 0)) return;
     int64_t s = std::min<int64_t>(256 / tail, kMaxTailSplits);
     s = std::min<int64_t>(s, (K / 64) / kMinSplitSteps);
     if (force > 0) s = std::min<int64_t>(force, K / 64);
@@ -457,6 +461,20 @@ static void tail_split_plan(int64_t tiles, int64_t K, int* tail_out, int* splits
 }
 static int64_t gemm_dtl_tail_workspace_bytes(int tail_tiles, int splits) {
     return (int64_t)tail_tiles * splits * (256 * 256 * 4);
+}
+
+// Few rows, long K: whether the 256x256 kernel with every tile's K loop split (the whole launch
+// treated as a partial round) beats the 128x128 kernel with its split.  Measured on N = 6656,
+// M = 256 / 512 / 1024 (26 / 52 / 104 tiles), caches flushed: row-major B wins from K = 4096 on
+// (M = 512, K = 16384: 200 -> 146 us; M = 1024, K = 32768: 622 -> 434 us) except 104 tiles at
+// K = 4096; transposed-contiguous B only with much work per tile (52 tiles at K = 32768
+// 308 -> 279 us, 104 tiles at K = 16384 287 -> 281 us; below that up to 15 % slower).
+static bool whole_launch_split_pays(int64_t M, int64_t N, int64_t K, bool b_nt) {
+    if (M <= 0 || N <= 0 || M % 256 != 0 || N % 256 != 0 || K % 64 != 0) return false;
+    const int64_t tiles = (M / 256) * (N / 256);
+    if (tiles < 24 || tiles > 128) return false;
+    if (b_nt) return tiles * K >= (int64_t)52 * 32768;
+    return K >= 8192 || (K >= 4096 && tiles <= 64);
 }
 
 // workspace of the two-pass form: S fp32 partial products of the whole [M, N] result
@@ -548,6 +566,12 @@ static int gemm_reduce(const void* A, int64_t lda_m, int64_t lda_k, const void* 
     // 256 CUs at once (512 tiles = 128 of the large ones): measured, the large tile is 15-30 %
     // faster from 144 tiles on and 5-10 % slower at 128, for K from 1024 to 8192.
     bool big = ((M + 255) / 256) * ((N + 255) / 256) > 128 && K >= 256;
+    // (few rows and a long K loop: the large tile again, with every tile's K loop split)
+    if (!big && workspace != nullptr && gather == nullptr && whole_launch_split_pays(M, N, K, b_nt)) {
+        int tail, ts;
+        tail_split_plan((M / 256) * (N / 256), K, &tail, &ts);
+        big = tail > 0 && gemm_dtl_tail_workspace_bytes(tail, ts) <= workspace_bytes;
+    }
     // KRAKEN_AMD_GEMM_TILE=128|256 overrides the choice (testing and tuning)
     if (const char* t = getenv("KRAKEN_AMD_GEMM_TILE")) {
         if (t[0] == '1') big = false;
@@ -688,7 +712,14 @@ extern "C" int64_t kr_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K) {
     }
     const int64_t tiles = ((M + 127) / 128) * ((N + 127) / 128);
     const int S = split_k_factor(tiles, K);
-    return S > 1 ? split_k_workspace_bytes(M, N, S) : 0;
+    int64_t bytes = S > 1 ? split_k_workspace_bytes(M, N, S) : 0;
+    // the layout of B is not known here: enough for either kernel
+    if (force_tile == nullptr && (whole_launch_split_pays(M, N, K, true) || whole_launch_split_pays(M, N, K, false))) {
+        int tail, ts;
+        tail_split_plan((M / 256) * (N / 256), K, &tail, &ts);
+        if (tail > 0) bytes = std::max(bytes, gemm_dtl_tail_workspace_bytes(tail, ts));
+    }
+    return bytes;
 }
 
 extern "C" int kr_gemm_reduce_ws_bf16(const void* A, int64_t lda_m, int64_t lda_k, const void* B, int64_t ldb_k,

@@ -532,7 +532,9 @@ hipError_t launch_gemm_dtl(const GemmArgs& g, bool b_nt, hipStream_t st, void* w
         if (e != hipSuccess) return e;
         opt_in[which] = true;
     }
-    if (b_nt) {
+    if (grid.x == 0) {
+        // every tile belongs to the split partial round
+    } else if (b_nt) {
         if (ragged) hipLaunchKernelGGL((gemm_dtl_kernel<true, true>), grid, block, LDS_BYTES, st, g);
         else hipLaunchKernelGGL((gemm_dtl_kernel<true, false>), grid, block, LDS_BYTES, st, g);
     } else {

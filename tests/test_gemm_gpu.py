@@ -428,6 +428,42 @@ def test_tail_round_split(dev, monkeypatch, b_t, force):
 
 
 @pytest.mark.parametrize("b_t", [False, True])
+def test_whole_launch_split_for_few_rows(dev, monkeypatch, b_t):
+    """24 tiles of 256 x 256 and a long K loop: no full round at all, every tile's K loop is
+    shared by 8 workgroups of the large-tile kernel.  Chosen by default for row-major B; forced
+    for transposed-contiguous B (which takes this path only with more work per tile)."""
+    M, N, K, W = 512, 3072, 8192, 4
+    lib = _lib.load()
+    if b_t:
+        monkeypatch.setenv("KRAKEN_AMD_GEMM_TILE", "256")
+    assert lib.kr_gemm_workspace_bytes(M, N, K) == 24 * 8 * 256 * 256 * 4
+    a, b, _ = mk(M, N, K, 0, b_t, seed=11)
+    ad, bd = a.to(dev), b.to(dev)
+    prod = a.float() @ b.float()
+    plain = fused.gemm_one_shot_all_reduce_fused(ad, bd)
+    torch.testing.assert_close(plain.cpu(), prod, rtol=1e-3, atol=2e-3)
+    assert torch.equal(plain, fused.gemm_one_shot_all_reduce_fused(ad, bd))          # reproducible
+    monkeypatch.setenv("KRAKEN_AMD_GEMM_TILE", "128")
+    other = fused.gemm_one_shot_all_reduce_fused(ad, bd)
+    monkeypatch.setenv("KRAKEN_AMD_GEMM_TILE", "256") if b_t else monkeypatch.delenv("KRAKEN_AMD_GEMM_TILE")
+    torch.testing.assert_close(plain, other, rtol=1e-4, atol=1e-4)
+    assert not torch.equal(plain, other)                                              # another kernel did run
+    peers = torch.stack([orc.randn_bf16((M, N), 100 + j) for j in range(2)])
+    bias = orc.randn_bf16((N,), 9, 0.02)
+    out = fused.gemm_one_shot_all_reduce_fused(ad, bd, peers=peers.to(dev), bias=bias.to(dev), out_dtype=BF16)
+    torch.testing.assert_close(out.cpu(), (prod + peers.float().sum(0) + bias.float()).to(BF16), **TOL)
+    rank = 1                                     # band = rows 128..255, inside the first row of tiles
+    bp = torch.stack([orc.randn_bf16((M // W, N), 200 + j) for j in range(W - 1)])
+    c_scratch = torch.zeros(M, N, dtype=BF16, device=dev)
+    out = fused.gemm_reduce_scatter(ad, bd, peers=bp.to(dev), rank=rank, world_size=W, c_scratch=c_scratch)
+    band = slice(rank * (M // W), (rank + 1) * (M // W))
+    torch.testing.assert_close(out.cpu(), (prod[band] + bp.float().sum(0)).to(BF16), **TOL)
+    rows = torch.ones(M, dtype=torch.bool)
+    rows[band] = False
+    torch.testing.assert_close(c_scratch.cpu()[rows], prod[rows].to(BF16), **TOL)
+
+
+@pytest.mark.parametrize("b_t", [False, True])
 def test_ragged_shapes_on_the_large_tile(dev, monkeypatch, b_t):
     """M and N that 256 does not divide, on the 256 x 256 kernel: edge tiles read short operand
     panels and store through the bounds-checked epilogue; every epilogue form."""
