@@ -392,13 +392,8 @@ static hipError_t launch_gemm(const GemmArgs& g, bool b_nt, bool even, hipStream
 #define KR_LAUNCH(NT, EV)                                                                             \
     do {                                                                                              \
         auto kfn = gemm_reduce_kernel<BM, BN, WM, WN, NT, EV>;                                        \
-        static bool lds_opt_in = false; /* benign race: the attribute call is idempotent */          \
-        if (!lds_opt_in) {                                                                            \
-            hipError_t e = hipFuncSetAttribute((const void*)kfn,                                      \
-                                               hipFuncAttributeMaxDynamicSharedMemorySize, LDS);      \
-            if (e != hipSuccess) return e;                                                            \
-            lds_opt_in = true;                                                                        \
-        }                                                                                             \
+        static std::atomic<uint64_t> opted{0};                                                        \
+        if (hipError_t e = lds_opt_in((const void*)kfn, LDS, opted); e != hipSuccess) return e;       \
         hipLaunchKernelGGL(kfn, grid, block, LDS, st, g);                                             \
     } while (0)
     if (b_nt) {

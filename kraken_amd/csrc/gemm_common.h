@@ -1,6 +1,7 @@
 // Pieces shared by the GEMM kernels: argument block, tile schedule, fused epilogue.
 #pragma once
 
+#include <atomic>
 #include <type_traits>
 
 #include "common.h"
@@ -40,6 +41,20 @@ struct GemmArgs {
     int group_n;         // column panels per scheduling group (tile_schedule)
     int peers_on_mfma;   // 256x256 kernel: add whole-band tiles' peers through the matrix cores
 };
+
+// Opt a kernel into more than 64 KiB of dynamic LDS, once per device: the attribute belongs to the
+// current device's copy of the code.  `done`: the call site's own bit mask of devices.
+inline hipError_t lds_opt_in(const void* fn, int bytes, std::atomic<uint64_t>& done) {
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return e;
+    const uint64_t bit = 1ull << (dev & 63);
+    if (done.load(std::memory_order_acquire) & bit) return hipSuccess;
+    e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+    if (e != hipSuccess) return e;
+    done.fetch_or(bit, std::memory_order_release);
+    return hipSuccess;
+}
 
 // LDS-DMA kernel for shapes the 256x256 tile divides (gemm_dtl.hip)
 bool gemm_dtl_supported(const GemmArgs& g);

@@ -525,13 +525,8 @@ hipError_t launch_gemm_dtl(const GemmArgs& g, bool b_nt, hipStream_t st, void* w
     const bool ragged = g.M % BM != 0 || g.N % BN != 0;
     const void* kfn = b_nt ? (ragged ? (const void*)gemm_dtl_kernel<true, true> : (const void*)gemm_dtl_kernel<true, false>)
                            : (ragged ? (const void*)gemm_dtl_kernel<false, true> : (const void*)gemm_dtl_kernel<false, false>);
-    static bool opt_in[4] = {false, false, false, false};   // benign race: the attribute call is idempotent
-    const int which = (b_nt ? 2 : 0) + (ragged ? 1 : 0);
-    if (!opt_in[which]) {
-        hipError_t e = hipFuncSetAttribute(kfn, hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES);
-        if (e != hipSuccess) return e;
-        opt_in[which] = true;
-    }
+    static std::atomic<uint64_t> opted[4];
+    if (hipError_t e = lds_opt_in(kfn, LDS_BYTES, opted[(b_nt ? 2 : 0) + (ragged ? 1 : 0)]); e != hipSuccess) return e;
     if (grid.x == 0) {
         // every tile belongs to the split partial round
     } else if (b_nt) {
@@ -544,15 +539,9 @@ hipError_t launch_gemm_dtl(const GemmArgs& g, bool b_nt, hipStream_t st, void* w
     if (g.tail_tiles > 0) {
         // the tiles of the last partial round: k_splits workgroups each, parts to the workspace,
         // then the sum and the epilogue
-        static bool split_opt_in[2] = {false, false};
-        if (!split_opt_in[b_nt]) {
-            hipError_t e = b_nt ? hipFuncSetAttribute((const void*)gemm_dtl_split_kernel<true>,
-                                                      hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES)
-                                : hipFuncSetAttribute((const void*)gemm_dtl_split_kernel<false>,
-                                                      hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES);
-            if (e != hipSuccess) return e;
-            split_opt_in[b_nt] = true;
-        }
+        static std::atomic<uint64_t> split_opted[2];
+        const void* sfn = b_nt ? (const void*)gemm_dtl_split_kernel<true> : (const void*)gemm_dtl_split_kernel<false>;
+        if (hipError_t e2 = lds_opt_in(sfn, LDS_BYTES, split_opted[b_nt]); e2 != hipSuccess) return e2;
         hipError_t e = hipGetLastError();
         if (e != hipSuccess) return e;
         GemmArgs gs = g;
