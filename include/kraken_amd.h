@@ -285,6 +285,44 @@ int kr_all_gather_matmul_bf16(const void* A, int64_t lda_m, const void* A_local,
 int kr_stream_write_value32(uint32_t* addr, uint32_t value, void* stream);
 
 /*
+ * Producer GEMM of the copy-engine reduce-scatter:  C[M,N] = A[M,K] @ B[K,N]  (bf16, fp32
+ * accumulate, bf16 result, every row written to C), announcing its progress per destination rank
+ * while it runs.  Rank r's band is rows [r*M/W, (r+1)*M/W) of C.  The order of the M tiles is
+ * rotated so that the band of rank+1 is finished first, then rank+2, ..., the own band last.
+ * A workgroup that has stored a tile adds 1 to progress[r] for every band r the tile's rows
+ * touch; the workgroup whose add completes band r (all column tiles of all row tiles that
+ * overlap the band) stores 1 to signal_pad[r].  When signal_pad[r] is 1, band r of C is complete
+ * and visible to a copy that is ordered behind the flag (kr_stream_wait_value32).
+ * progress and signal_pad: uint32[W] in device memory, 4-byte aligned, zeroed by the caller
+ * before the call.  The count a band reaches depends on the kernel's tile size (128 or 256
+ * rows); only signal_pad is meant to be waited on.  M % W == 0, 0 <= rank < W, K % 8 == 0,
+ * N % 8 == 0; M == 0 or N == 0: nothing is launched and no flag is set.
+ * A, B as for kr_gemm_reduce_bf16.
+ *
+ * Replaces kraken/fused/gemm_reduce_scatter_ce_persistent.py:46-134
+ * (_gemm_producer_persistent_kernel: tile order :88,102, progress counters and signals :117-132)
+ * as launched by gemm_producer_w_progress (:178-242).
+ */
+int kr_gemm_producer_bf16(const void* A, int64_t lda_m, int64_t lda_k,
+                          const void* B, int64_t ldb_k, int64_t ldb_n,
+                          int64_t M, int64_t N, int64_t K,
+                          void* C, int W, int rank,
+                          uint32_t* progress, uint32_t* signal_pad, void* stream);
+
+/*
+ * Stream-ordered wait: what is enqueued on `stream` behind this call starts once *addr == value
+ * (a one-wave kernel that polls the word at system scope).  The wait is bounded: after
+ * wait_limit_us microseconds (0: 5 s) the kernel stores 1 to *status (device int32, may be NULL)
+ * and ends all the same, so the stream always drains; the caller checks status afterwards.
+ * The writer must already be enqueued on another stream, or the wait runs to its limit.
+ * Replaces driver.cuStreamWaitValue32(stream, addr, 1, CU_STREAM_WAIT_VALUE_EQ) in front of
+ * every band copy of copy_engine_scatter
+ * (kraken/fused/gemm_reduce_scatter_ce_persistent.py:153-163).
+ */
+int kr_stream_wait_value32(const uint32_t* addr, uint32_t value, int64_t wait_limit_us,
+                           int32_t* status, void* stream);
+
+/*
  * Tile reduce of the copy-engine reduce-scatter variant: `in` is [W*rows, N]
  * bf16 (band r holds what rank r pushed), and
  *   out[m, n] = sum_{i=0..W-1} in[((i + rank + 1) % W) * rows + m, n]

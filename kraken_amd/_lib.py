@@ -80,6 +80,12 @@ _SIGNATURES = {
          c_int, c_int, c_int, c_void_p, c_int64, c_void_p, c_void_p, c_void_p],
     ),
     "kr_stream_write_value32": (c_int, [c_void_p, ctypes.c_uint32, c_void_p]),
+    "kr_gemm_producer_bf16": (
+        c_int,
+        [c_void_p, c_int64, c_int64, c_void_p, c_int64, c_int64, c_int64, c_int64, c_int64, c_void_p,
+         c_int, c_int, c_void_p, c_void_p, c_void_p],
+    ),
+    "kr_stream_wait_value32": (c_int, [c_void_p, ctypes.c_uint32, c_int64, c_void_p, c_void_p]),
     "kr_reduce_rotated_bf16": (c_int, [c_void_p, c_int, c_int64, c_int64, c_int, c_int, c_void_p, c_void_p]),
 }
 

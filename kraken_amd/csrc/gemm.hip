@@ -475,7 +475,9 @@ static bool whole_launch_split_pays(int64_t M, int64_t N, int64_t K, bool b_nt) 
 // workspace of the two-pass form: S fp32 partial products of the whole [M, N] result
 static int64_t split_k_workspace_bytes(int64_t M, int64_t N, int S) { return (int64_t)S * M * N * 4; }
 
-// Arrival flags of the all-gather matmul (null pointer to gemm_reduce: A is complete).
+// What the kernel exchanges with other streams while it runs (null pointer to gemm_reduce:
+// nothing): the arrival flags of the all-gather matmul (progress == nullptr: A is complete) and
+// the per-band counters of the producer GEMM (band_counter == nullptr: none).
 struct GatherSpec {
     const void* a_local;
     int64_t lda_local;
@@ -484,6 +486,9 @@ struct GatherSpec {
     int64_t comm_rows;
     int64_t wait_limit_us;
     int* status;
+    uint32_t* band_counter;
+    uint32_t* band_signal;
+    int64_t count_rows;
 };
 
 // Everything of the entry points except the peers: argument checks in the documented
@@ -547,6 +552,14 @@ static int gemm_reduce(const void* A, int64_t lda_m, int64_t lda_k, const void* 
         g.wait_ticks = (uint64_t)gather->wait_limit_us * 100u;   // 100 MHz constant clock
         g.status = gather->status;
     }
+    g.band_counter = nullptr;
+    g.band_signal = nullptr;
+    g.count_rows = 1;
+    if (gather != nullptr && gather->band_counter != nullptr) {
+        g.band_counter = gather->band_counter;
+        g.band_signal = gather->band_signal;
+        g.count_rows = (int)gather->count_rows;
+    }
     g.bias = (const uint16_t*)bias;
     g.band_row0 = (int)band_row0;
     g.band_rows = (int)band_rows;
@@ -593,7 +606,10 @@ static int gemm_reduce(const void* A, int64_t lda_m, int64_t lda_k, const void* 
     // walks spans all row blocks in the order of their arrival (every XCD then starts on the
     // local shard and waits little); with wide groups the XCDs that own the last blocks idle
     // until those have arrived.
-    if (g.progress != nullptr) g.group_n = (g.tiles_n + kXcds - 1) / kXcds;
+    // The same for row bands that are flagged as they complete: every XCD then moves from band to
+    // band in the order of the destinations, and a band is complete once all eight have passed it
+    // (with wide groups every band would only be complete when the last group is).
+    if (g.progress != nullptr || g.band_counter != nullptr) g.group_n = (g.tiles_n + kXcds - 1) / kXcds;
     if (const char* t = getenv("KRAKEN_AMD_GEMM_GROUP")) {
         const int v = atoi(t);
         if (v >= 1 && v <= 64) g.group_n = v;
@@ -678,7 +694,7 @@ extern "C" int kr_all_gather_matmul_bf16(const void* A, int64_t lda_m, const voi
     if (A_local != nullptr && lda_local < K) return KR_ERR_LAYOUT;
     if ((reinterpret_cast<uintptr_t>(progress) & 3u) != 0 || (reinterpret_cast<uintptr_t>(status) & 3u) != 0)
         return KR_ERR_ALIGNMENT;
-    GatherSpec gs;
+    GatherSpec gs{};
     gs.a_local = A_local;
     gs.lda_local = lda_local;
     gs.local_rows = M / W;
@@ -690,6 +706,24 @@ extern "C" int kr_all_gather_matmul_bf16(const void* A, int64_t lda_m, const voi
     // no reduce: the band is every row, no peers, no bias; tile order rotated to the local shard
     return gemm_reduce(A, lda_m, 1, B, ldb_k, ldb_n, M, N, K, nullptr, 0, nullptr, 0, nullptr, 0, M, nullptr, C, 0,
                        gs.local_row0, stream, &gs);
+}
+
+extern "C" int kr_gemm_producer_bf16(const void* A, int64_t lda_m, int64_t lda_k, const void* B, int64_t ldb_k,
+                                     int64_t ldb_n, int64_t M, int64_t N, int64_t K, void* C, int W, int rank,
+                                     uint32_t* progress, uint32_t* signal_pad, void* stream) {
+    if (W < 1 || W > KR_MAX_WORLD) return KR_ERR_WORLD_SIZE;
+    if (rank < 0 || rank >= W) return KR_ERR_BAND;
+    if (M < 0 || M % W != 0) return KR_ERR_BAD_DIM;
+    if (progress == nullptr || signal_pad == nullptr || (M > 0 && N > 0 && C == nullptr)) return KR_ERR_NULL_POINTER;
+    if ((reinterpret_cast<uintptr_t>(progress) & 3u) != 0 || (reinterpret_cast<uintptr_t>(signal_pad) & 3u) != 0)
+        return KR_ERR_ALIGNMENT;
+    GatherSpec ps{};
+    ps.band_counter = progress;
+    ps.band_signal = signal_pad;
+    ps.count_rows = M > 0 ? M / W : 1;
+    // no reduce band: every row of C goes to `C`; tile order rotated to the band of rank + 1
+    return gemm_reduce(A, lda_m, lda_k, B, ldb_k, ldb_n, M, N, K, nullptr, 0, nullptr, 0, nullptr, 0, 0, C, nullptr,
+                       0, ((int64_t)(rank + 1) % W) * (M / W), stream, &ps);
 }
 
 extern "C" int64_t kr_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K) {

@@ -40,6 +40,11 @@ struct GemmArgs {
     int tail_tiles;
     int group_n;         // column panels per scheduling group (tile_schedule)
     int peers_on_mfma;   // 256x256 kernel: add whole-band tiles' peers through the matrix cores
+    // producer of the copy-engine reduce-scatter (band_counter == nullptr: off): finished tiles are
+    // counted per destination rank, whose band is count_rows rows of C
+    uint32_t* band_counter;   // [M / count_rows] tiles finished that touch the band
+    uint32_t* band_signal;    // [M / count_rows] set to 1 by the workgroup that finishes the band's last tile
+    int count_rows;
 };
 
 // Opt a kernel into more than 64 KiB of dynamic LDS, once per device: the attribute belongs to the
@@ -405,6 +410,31 @@ __device__ __forceinline__ void gemm_epilogue_impl(const GemmArgs& g, const int 
     }
 }
 
+// Producer side of the copy-engine reduce-scatter, called by the whole workgroup once its tile
+// (rows m0 .. m0+bm-1) is stored (kraken/fused/gemm_reduce_scatter_ce_persistent.py:117-132):
+// the tile is counted into the counter of every destination rank whose band of g.count_rows rows
+// it touches, and the workgroup whose count completes a band (all column tiles of all row tiles
+// that overlap it) sets the band's flag, on which a stream-ordered wait in front of the band's
+// copy is parked.  Order: every wave's stores are complete at the barrier; thread 0's release
+// fence then writes them back to memory before its count becomes visible, and the workgroup that
+// sees the last count acquires the others' before it publishes the flag.
+__device__ __forceinline__ void count_finished_tile(const GemmArgs& g, int m0, int bm) {
+    __syncthreads();
+    if (threadIdx.x != 0) return;
+    __atomic_thread_fence(__ATOMIC_RELEASE);   // system scope
+    const int m_last = min(m0 + bm, g.M) - 1;
+    for (int r = m0 / g.count_rows; r <= m_last / g.count_rows; ++r) {
+        const int t_lo = (int)(((int64_t)r * g.count_rows) / bm);
+        const int t_hi = (int)(((int64_t)(r + 1) * g.count_rows - 1) / bm);
+        const uint32_t band_tiles = (uint32_t)(t_hi - t_lo + 1) * (uint32_t)g.tiles_n;
+        const uint32_t before = __hip_atomic_fetch_add(g.band_counter + r, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (before + 1 == band_tiles) {
+            __atomic_thread_fence(__ATOMIC_ACQ_REL);
+            __hip_atomic_store(g.band_signal + r, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+        }
+    }
+}
+
 // n_peers and bias are what is still to be added here (a kernel that has already put the
 // peers or the bias into the accumulators passes 0 / nullptr); g is only read, never copied,
 // so the peer table stays in kernel-argument memory.
@@ -414,6 +444,7 @@ __device__ __forceinline__ void gemm_epilogue(const GemmArgs& g, int n_peers, co
                                               int m0, int n0, int wm, int wn, int lane, int wave) {
     if (g.out_is_fp32) gemm_epilogue_impl<true, BM, WTM, WTN, TM, TN, EVEN, EP_WAVE>(g, n_peers, bias, acc, smem, m0, n0, wm, wn, lane, wave);
     else gemm_epilogue_impl<false, BM, WTM, WTN, TM, TN, EVEN, EP_WAVE>(g, n_peers, bias, acc, smem, m0, n0, wm, wn, lane, wave);
+    if (g.band_counter != nullptr) count_finished_tile(g, m0, BM);
 }
 
 }  // namespace kr

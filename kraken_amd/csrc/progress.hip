@@ -11,11 +11,41 @@ __global__ __launch_bounds__(kWave) void write_value32_kernel(uint32_t* addr, ui
     if (threadIdx.x == 0) __hip_atomic_store(addr, value, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
 }
 
+// Stream-ordered wait: ends once *addr == value.  One lane polls with system-scope loads and a
+// short sleep; the wait is bounded by `ticks` of the 100 MHz constant clock, after which 1 is
+// stored to *status (if given) and the kernel ends all the same, so the stream always drains.
+// The acquire fence orders what follows on the stream behind the value seen.
+__global__ __launch_bounds__(kWave) void wait_value32_kernel(const uint32_t* addr, uint32_t value, uint64_t ticks,
+                                                             int* status) {
+    if (threadIdx.x != 0) return;
+    const uint64_t t0 = __builtin_amdgcn_s_memrealtime();
+    while (__hip_atomic_load(addr, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM) != value) {
+        if (__builtin_amdgcn_s_memrealtime() - t0 > ticks) {
+            if (status != nullptr) __hip_atomic_store(status, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+            break;
+        }
+        __builtin_amdgcn_s_sleep(32);
+    }
+    __atomic_thread_fence(__ATOMIC_ACQUIRE);
+}
+
 }  // namespace kr
 
 extern "C" int kr_stream_write_value32(uint32_t* addr, uint32_t value, void* stream) {
     if (addr == nullptr) return KR_ERR_NULL_POINTER;
     if ((reinterpret_cast<uintptr_t>(addr) & 3u) != 0) return KR_ERR_ALIGNMENT;
     hipLaunchKernelGGL(kr::write_value32_kernel, dim3(1), dim3(kr::kWave), 0, (hipStream_t)stream, addr, value);
+    return (int)hipGetLastError();
+}
+
+extern "C" int kr_stream_wait_value32(const uint32_t* addr, uint32_t value, int64_t wait_limit_us, int* status,
+                                      void* stream) {
+    if (addr == nullptr) return KR_ERR_NULL_POINTER;
+    if ((reinterpret_cast<uintptr_t>(addr) & 3u) != 0 || (reinterpret_cast<uintptr_t>(status) & 3u) != 0)
+        return KR_ERR_ALIGNMENT;
+    if (wait_limit_us < 0) return KR_ERR_BAD_DIM;
+    const uint64_t ticks = (uint64_t)(wait_limit_us > 0 ? wait_limit_us : 5000000) * 100u;   // default 5 s
+    hipLaunchKernelGGL(kr::wait_value32_kernel, dim3(1), dim3(kr::kWave), 0, (hipStream_t)stream, addr, value, ticks,
+                       status);
     return (int)hipGetLastError();
 }

@@ -185,6 +185,35 @@ def test_all_gather_matmul_argument_errors(lib):
     assert g(FAKE + 2, 1, None) == _lib.KR_ERR_ALIGNMENT
 
 
+def test_gemm_producer_argument_errors(lib):
+    f = lib.kr_gemm_producer_bf16
+    def args(**kw):
+        a = dict(A=FAKE, lda_m=64, lda_k=1, B=FAKE, ldb_k=64, ldb_n=1, M=512, N=64, K=64, C=FAKE, W=4, rank=1,
+                 progress=FAKE, signal=FAKE, stream=None)
+        a.update(kw)
+        return tuple(a.values())
+    assert f(*args(W=0)) == _lib.KR_ERR_WORLD_SIZE
+    assert f(*args(W=17)) == _lib.KR_ERR_WORLD_SIZE
+    assert f(*args(rank=4)) == _lib.KR_ERR_BAND
+    assert f(*args(rank=-1)) == _lib.KR_ERR_BAND
+    assert f(*args(M=510)) == _lib.KR_ERR_BAD_DIM             # 510 rows do not split into 4 bands
+    assert f(*args(progress=None)) == _lib.KR_ERR_NULL_POINTER
+    assert f(*args(signal=None)) == _lib.KR_ERR_NULL_POINTER
+    assert f(*args(C=None)) == _lib.KR_ERR_NULL_POINTER
+    assert f(*args(progress=FAKE + 2)) == _lib.KR_ERR_ALIGNMENT
+    assert f(*args(signal=FAKE + 1)) == _lib.KR_ERR_ALIGNMENT
+    assert f(*args(A=None)) == _lib.KR_ERR_NULL_POINTER
+    assert f(*args(K=60)) == _lib.KR_ERR_NUMEL_MOD8
+    assert f(*args(lda_k=2)) == _lib.KR_ERR_LAYOUT
+    assert f(*args(C=FAKE + 8)) == _lib.KR_ERR_ALIGNMENT
+    assert f(*args(M=0)) == 0                                 # nothing to compute, nothing launched
+    g = lib.kr_stream_wait_value32
+    assert g(None, 1, 0, None, None) == _lib.KR_ERR_NULL_POINTER
+    assert g(FAKE + 2, 1, 0, None, None) == _lib.KR_ERR_ALIGNMENT
+    assert g(FAKE, 1, 0, FAKE + 1, None) == _lib.KR_ERR_ALIGNMENT
+    assert g(FAKE, 1, -5, None, None) == _lib.KR_ERR_BAD_DIM
+
+
 def test_gemm_workspace_entries(lib):
     assert lib.kr_gemm_workspace_bytes(0, 128, 128) == 0
     assert lib.kr_gemm_workspace_bytes(8192, 8192, 8192) == 0

@@ -199,6 +199,96 @@ def test_ce_persistent_variant(dev, tile):
         torch.testing.assert_close(out.cpu(), want, **TOL)
 
 
+def _band_tile_counts(M, N, W, bm):
+    rows = M // W
+    return [(((r + 1) * rows - 1) // bm - (r * rows) // bm + 1) * -(-N // bm) for r in range(W)]
+
+
+@pytest.mark.parametrize("shape,W,rank", [((512, 256, 128), 4, 1), ((768, 384, 192), 3, 2), ((1024, 512, 256), 8, 7),
+                                          ((1000, 264, 512), 4, 0), ((1000, 264, 520), 4, 3)])
+def test_producer_gemm_flags_every_band(dev, tile, shape, W, rank):
+    """Producer GEMM of the copy-engine reduce-scatter: all of C, one counter and one flag per
+    destination rank's band (bands that start inside a tile included)."""
+    from kraken_amd.fused.gemm_reduce_scatter_ce_persistent import gemm_producer_w_progress
+    M, N, K = shape
+    a, b, _ = mk(M, N, K, 0, True, seed=W)
+    gemm_out = torch.full((M, N), float("nan"), dtype=BF16, device=dev)
+    progress = torch.zeros(W, dtype=torch.int32, device=dev)
+    signal_pad = torch.zeros(W, dtype=torch.int32, device=dev)
+    gemm_producer_w_progress(a.to(dev), b.to(dev), gemm_out, progress, signal_pad, {"RANK": rank, "WORLD_SIZE": W})
+    torch.cuda.synchronize()
+    assert signal_pad.tolist() == [1] * W
+    assert progress.tolist() in (_band_tile_counts(M, N, W, 128), _band_tile_counts(M, N, W, 256))
+    torch.testing.assert_close(gemm_out.cpu(), (a.float() @ b.float()).to(BF16), **TOL)
+
+
+@pytest.mark.parametrize("rank", [0, 2])
+def test_copy_engine_scatter_overlaps_the_producer(dev, tile, rank):
+    """The reference's overlap: the band copies sit on a side stream behind stream-ordered waits
+    for the producer's flags (kraken/fused/gemm_reduce_scatter_ce_persistent.py:137-175,343-370)."""
+    from kraken_amd.fused.gemm_reduce_scatter_ce_persistent import gemm_producer_w_progress
+    M, N, K, W = 2048, 1024, 256, 4
+    a, b, _ = mk(M, N, K, 0, True, seed=3)
+    peers = torch.stack([orc.randn_bf16((M // W, N), 100 + j) for j in range(W - 1)])
+    sent = torch.full((W, M // W, N), float("nan"), dtype=BF16, device=dev)
+    status = torch.zeros(1, dtype=torch.int32, device=dev)
+    out = fused.gemm_reduce_scatter_ce_persistent(a.to(dev), b.to(dev), peers=peers.to(dev), rank=rank, sent=sent,
+                                                  status=status)
+    torch.cuda.synchronize()
+    assert status.item() == 0
+    c = (a.float() @ b.float()).to(BF16)
+    bands = list(peers)
+    bands.insert(rank, c[rank * M // W:(rank + 1) * M // W])
+    want = orc.reduce_rotated(torch.cat(bands, 0), W, rank, acc_bf16=True)
+    torch.testing.assert_close(out.cpu(), want, **TOL)
+    # every other rank's band went out as the GEMM wrote it; the own band went to the scatter buffer
+    gemm_out = torch.empty(M, N, dtype=BF16, device=dev)
+    progress = torch.zeros(W, dtype=torch.int32, device=dev)
+    signal_pad = torch.zeros(W, dtype=torch.int32, device=dev)
+    gemm_producer_w_progress(a.to(dev), b.to(dev), gemm_out, progress, signal_pad, {"RANK": rank, "WORLD_SIZE": W})
+    for r in range(W):
+        if r != rank:
+            assert torch.equal(sent[r], gemm_out[r * M // W:(r + 1) * M // W])
+        else:
+            assert torch.isnan(sent[r].float()).all()
+    assert torch.equal(out, fused.gemm_reduce_scatter_ce_persistent(a.to(dev), b.to(dev), peers=peers.to(dev), rank=rank))
+
+
+def test_copy_engine_scatter_wait_is_bounded(dev):
+    """A flag that never comes: the stream-ordered wait gives up after its limit, records it in
+    `status`, and the stream drains."""
+    from kraken_amd.fused.gemm_reduce_scatter_ce_persistent import copy_engine_scatter
+    W, rows, N = 2, 64, 128
+    inp = torch.ones(W * rows, N, dtype=BF16, device=dev)
+    signal_pad = torch.tensor([1, 0], dtype=torch.int32, device=dev)      # band 1 is never flagged
+    status = torch.zeros(1, dtype=torch.int32, device=dev)
+    outs = [torch.zeros(rows, N, dtype=BF16, device=dev) for _ in range(W)]
+    copy_engine_scatter(inp, outs, signal_pad, rank=0, wait_limit_us=2000, status=status)
+    torch.cuda.synchronize()
+    assert status.item() == 1
+    ok = torch.zeros(1, dtype=torch.int32, device=dev)
+    copy_engine_scatter(inp, [outs[0], None], torch.ones(W, dtype=torch.int32, device=dev), rank=1,
+                        wait_limit_us=2000, status=ok)
+    torch.cuda.synchronize()
+    assert ok.item() == 0 and torch.equal(outs[0], inp[:rows])
+
+
+def test_ce_persistent_reference_shape(dev):
+    """(8192, 4096, 14336), the shape of test/test_gemm_reduce_scatter.py:93-111 (tolerance 1e-2
+    there; the gate here is the library's 2e-2 on sampled rows)."""
+    M, N, K, W, rank = 8192, 4096, 14336, 8, 5
+    a = orc.randn_bf16((M, K), 42)
+    b = orc.randn_bf16((N, K), 43, 0.02).T
+    peers = torch.stack([orc.randn_bf16((M // W, N), 100 + j) for j in range(W - 1)])
+    out = fused.gemm_reduce_scatter_ce_persistent(a.to(dev), b.to(dev), peers=peers.to(dev), rank=rank)
+    pick = torch.tensor([0, 1, 127, 128, 255, 256, 700, 1023])
+    own = (a[rank * 1024 + pick].float() @ b.float()).to(BF16)
+    bands = [p[pick] for p in peers]
+    bands.insert(rank, own)
+    want = orc.reduce_rotated(torch.cat(bands, 0), W, rank, acc_bf16=True)
+    torch.testing.assert_close(out.cpu()[pick], want, **TOL)
+
+
 def _sampled_rows_check(got, rows, a, b, extra, tol=TOL):
     want = a[rows].float() @ b.float()
     if extra is not None:
