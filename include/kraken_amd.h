@@ -323,6 +323,17 @@ int kr_stream_wait_value32(const uint32_t* addr, uint32_t value, int64_t wait_li
                            int32_t* status, void* stream);
 
 /*
+ * Stream-ordered device-to-device copy of `bytes` bytes that runs on the GPU's copy engines
+ * (SDMA) and not as a copy kernel, so it takes no compute units from a GEMM running beside it.
+ * Source and destination must not overlap.  bytes == 0: nothing is done.
+ * Replaces the `.copy_()` calls that the reference issues on its backend stream for the copy
+ * engines: the chunk copies of the all-gather (kraken/comm/copy_engine_all_gather.py:44-46) and
+ * the band copies of copy_engine_scatter
+ * (kraken/fused/gemm_reduce_scatter_ce_persistent.py:165-169).
+ */
+int kr_copy_engine_memcpy(void* dst, const void* src, int64_t bytes, void* stream);
+
+/*
  * Tile reduce of the copy-engine reduce-scatter variant: `in` is [W*rows, N]
  * bf16 (band r holds what rank r pushed), and
  *   out[m, n] = sum_{i=0..W-1} in[((i + rank + 1) % W) * rows + m, n]

@@ -86,6 +86,7 @@ _SIGNATURES = {
          c_int, c_int, c_void_p, c_void_p, c_void_p],
     ),
     "kr_stream_wait_value32": (c_int, [c_void_p, ctypes.c_uint32, c_int64, c_void_p, c_void_p]),
+    "kr_copy_engine_memcpy": (c_int, [c_void_p, c_void_p, c_int64, c_void_p]),
     "kr_reduce_rotated_bf16": (c_int, [c_void_p, c_int, c_int64, c_int64, c_int, c_int, c_void_p, c_void_p]),
 }
 
@@ -158,3 +159,12 @@ def ptr(t: torch.Tensor | None) -> int | None:
 
 def current_stream(dev: torch.device) -> int:
     return torch.cuda.current_stream(dev).cuda_stream
+
+
+def copy_engine_copy(dst: torch.Tensor, src: torch.Tensor, stream: int) -> None:
+    """``dst.copy_(src)`` on the copy engines (``kr_copy_engine_memcpy``): both contiguous,
+    same dtype and number of elements, on the stream given (a raw ``hipStream_t``)."""
+    assert dst.is_contiguous() and src.is_contiguous() and dst.dtype == src.dtype and dst.numel() == src.numel()
+    rc = load().kr_copy_engine_memcpy(dst.data_ptr(), src.data_ptr(), src.numel() * src.element_size(), stream)
+    check(rc, "copy_engine_memcpy")
+

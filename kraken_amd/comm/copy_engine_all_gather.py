@@ -30,6 +30,7 @@ def _copy_engine_all_gather_w_progress(
     backend_stream: torch.cuda.Stream | None = None,
     *,
     rank: int = 0,
+    copy_engine: bool = False,
 ) -> torch.cuda.Stream:
     """Copy the W shards into ``output`` chunk by chunk on a side stream, flagging each chunk.
 
@@ -42,8 +43,10 @@ def _copy_engine_all_gather_w_progress(
     ``output`` and then ``progress[chunk]`` is set to 1 by a stream-ordered
     flag write (``:47-53``).  The side stream first waits for the current
     stream (``:35``); the caller makes the current stream wait for the returned
-    stream when it needs the gathered tensor (``:118``).  The copies are plain
-    device-to-device copies; ``progress`` must have been zeroed on the current
+    stream when it needs the gathered tensor (``:118``).  The copies are ordinary
+    device-to-device copy kernels; ``copy_engine=True`` hands them to the GPU's
+    copy engines (``kr_copy_engine_memcpy``), which take no compute units but
+    are slower within one GPU.  ``progress`` must have been zeroed on the current
     stream beforehand.
     """
     peers = PeerBuffers(inp)
@@ -69,7 +72,11 @@ def _copy_engine_all_gather_w_progress(
             src = peers.slice(src_rank).reshape(-1)
             for split_id in range(splits_per_rank):
                 c = src_rank * splits_per_rank + split_id
-                flat_out[c * chunk:(c + 1) * chunk].copy_(src[split_id * chunk:(split_id + 1) * chunk])
+                dst_c, src_c = flat_out[c * chunk:(c + 1) * chunk], src[split_id * chunk:(split_id + 1) * chunk]
+                if copy_engine:
+                    _lib.copy_engine_copy(dst_c, src_c, backend_stream.cuda_stream)
+                else:
+                    dst_c.copy_(src_c)
                 rc = lib.kr_stream_write_value32(progress.data_ptr() + 4 * c, 1, backend_stream.cuda_stream)
                 _lib.check(rc, "stream_write_value32")
     return backend_stream
@@ -83,7 +90,7 @@ def all_gather_w_progress(a_shared, a_out: torch.Tensor | None = None, progress:
     (``kraken/comm/copy_engine_all_gather.py:63-120``): allocates ``a_out`` and
     ``progress`` when not given, zeroes ``progress`` (``:108``), runs the chunked
     copy on the side stream and makes the current stream wait for it.  kwargs:
-    ``splits_per_rank`` (default 1), ``rank`` (default 0).
+    ``splits_per_rank`` (default 1), ``rank`` (default 0), ``copy_engine`` (default False).
     """
     peers = PeerBuffers(a_shared)
     splits = kwargs.get("splits_per_rank", 1)
@@ -97,6 +104,7 @@ def all_gather_w_progress(a_shared, a_out: torch.Tensor | None = None, progress:
         progress = torch.zeros(peers.W * splits, dtype=torch.int32, device=dev)
     else:
         progress.fill_(0)
-    stream = _copy_engine_all_gather_w_progress(a_out, a_shared, progress, splits, rank=rank)
+    stream = _copy_engine_all_gather_w_progress(a_out, a_shared, progress, splits, rank=rank,
+                                                copy_engine=kwargs.get("copy_engine", False))
     torch.cuda.current_stream(dev).wait_stream(stream)
     return a_out

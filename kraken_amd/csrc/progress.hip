@@ -1,4 +1,5 @@
-// Stream-ordered 32-bit flag write: the arrival signal behind a chunk copy of the all-gather.
+// Stream-ordered flag write and flag wait, and the copy-engine copy they bracket: the pieces of
+// the overlap of copies with a running GEMM (all-gather matmul, copy-engine reduce-scatter).
 #include "common.h"
 
 namespace kr {
@@ -48,4 +49,13 @@ extern "C" int kr_stream_wait_value32(const uint32_t* addr, uint32_t value, int6
     hipLaunchKernelGGL(kr::wait_value32_kernel, dim3(1), dim3(kr::kWave), 0, (hipStream_t)stream, addr, value, ticks,
                        status);
     return (int)hipGetLastError();
+}
+
+extern "C" int kr_copy_engine_memcpy(void* dst, const void* src, int64_t bytes, void* stream) {
+    if (bytes < 0) return KR_ERR_BAD_DIM;
+    if (bytes == 0) return KR_OK;
+    if (dst == nullptr || src == nullptr) return KR_ERR_NULL_POINTER;
+    // a device-to-device copy that the runtime hands to the copy engines instead of a copy kernel:
+    // it takes no CUs from the GEMM that runs beside it
+    return (int)hipMemcpyAsync(dst, src, (size_t)bytes, hipMemcpyDeviceToDeviceNoCU, (hipStream_t)stream);
 }

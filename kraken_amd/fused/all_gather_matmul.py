@@ -65,6 +65,8 @@ def all_gather_matmul(
       (``:95-110``).  The current stream then waits for the side stream
       (``:316``).  ``status`` (int32 ``[1]``, zeroed by the caller) receives a
       non-zero value if a tile's wait ran out (``wait_limit_us``, default 5 s).
+      The copies are ordinary copy kernels, which share the compute units with
+      the GEMM; ``copy_engine=True`` hands them to the GPU's copy engines.
 
     In both modes the order of the M tiles is rotated so that the shard of
     ``rank`` (kwarg, default 0) is consumed first and the others in the order
@@ -114,7 +116,8 @@ def all_gather_matmul(
         progress = torch.zeros(W * splits, dtype=torch.int32, device=dev)
     else:
         progress.fill_(0)
-    backend_stream = _copy_engine_all_gather_w_progress(a_out, a_shared, progress, splits, rank=rank)
+    backend_stream = _copy_engine_all_gather_w_progress(a_out, a_shared, progress, splits, rank=rank,
+                                                        copy_engine=kwargs.get("copy_engine", False))
     configs = {"RANK": rank, "WORLD_SIZE": W, "SPLITS_PER_RANK": splits,
                "wait_limit_us": kwargs.get("wait_limit_us", 0)}
     c = _matmul_w_progress(a_out, peers.slice(rank), b, progress, configs, kwargs.get("status"))

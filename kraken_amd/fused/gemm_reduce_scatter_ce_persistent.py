@@ -83,6 +83,7 @@ def copy_engine_scatter(
     rank: int = 0,
     wait_limit_us: int = 0,
     status: torch.Tensor | None = None,
+    copy_engine: bool = False,
 ) -> None:
     """Copy every finished band of ``inp [M, N]`` to its destination, on the current stream.
 
@@ -95,7 +96,9 @@ def copy_engine_scatter(
     a sequence of W tensors ``[M/W, N]`` (``None`` entries are skipped: no wait, no
     copy); ``output[r]`` stands for slot ``rank`` of rank r's symmetric buffer
     (``:165-169``).  The waits are bounded (``wait_limit_us``, default 5 s); a wait
-    that runs out sets ``status`` (int32 ``[1]``, zeroed by the caller) to 1.
+    that runs out sets ``status`` (int32 ``[1]``, zeroed by the caller) to 1.  The
+    copies are ordinary copy kernels; ``copy_engine=True`` hands them to the GPU's
+    copy engines (``kr_copy_engine_memcpy``).
     """
     M, N = inp.shape
     W = len(output)
@@ -113,7 +116,11 @@ def copy_engine_scatter(
         assert tuple(dst.shape) == (m_per_rank, N) and dst.dtype == inp.dtype
         rc = lib.kr_stream_wait_value32(signal_pad.data_ptr() + 4 * remote, 1, wait_limit_us, _lib.ptr(status), stream)
         _lib.check(rc, "stream_wait_value32")
-        dst.copy_(inp[remote * m_per_rank:(remote + 1) * m_per_rank])
+        band = inp[remote * m_per_rank:(remote + 1) * m_per_rank]
+        if copy_engine and dst.is_contiguous() and band.is_contiguous():
+            _lib.copy_engine_copy(dst, band, stream)
+        else:
+            dst.copy_(band)
 
 
 def gemm_reduce_scatter_ce_persistent(
@@ -140,7 +147,7 @@ def gemm_reduce_scatter_ce_persistent(
     stream while the GEMM runs.  The current stream then waits for the side stream
     (``:370``) and the reduce sums the W bands starting at ``rank + 1``
     (``:258-279``).  kwargs ``rank`` (default 0), ``world_size``, ``fp32_acc``,
-    ``wait_limit_us``, ``status``.
+    ``wait_limit_us``, ``status``, ``copy_engine``.
     """
     assert reduce_op == "sum", "only support sum for now"
     assert a.dtype == torch.bfloat16 and b.dtype == torch.bfloat16, "Only bfloat16 is supported for now."
@@ -180,7 +187,8 @@ def gemm_reduce_scatter_ce_persistent(
                 scatter_out[r].copy_(peers[j])
         if sent is not None:
             copy_engine_scatter(gemm_out, dests, signal_pad, rank=rank,
-                                wait_limit_us=kwargs.get("wait_limit_us", 0), status=kwargs.get("status"))
+                                wait_limit_us=kwargs.get("wait_limit_us", 0), status=kwargs.get("status"),
+                                copy_engine=kwargs.get("copy_engine", False))
     if sent is None:
         # only the own band has a destination on this GPU, and it is the last one the GEMM
         # finishes: its copy gains nothing from a flag and goes behind the GEMM in stream order

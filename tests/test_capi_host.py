@@ -212,6 +212,11 @@ def test_gemm_producer_argument_errors(lib):
     assert g(FAKE + 2, 1, 0, None, None) == _lib.KR_ERR_ALIGNMENT
     assert g(FAKE, 1, 0, FAKE + 1, None) == _lib.KR_ERR_ALIGNMENT
     assert g(FAKE, 1, -5, None, None) == _lib.KR_ERR_BAD_DIM
+    h = lib.kr_copy_engine_memcpy
+    assert h(FAKE, FAKE + 64, -1, None) == _lib.KR_ERR_BAD_DIM
+    assert h(None, None, 0, None) == 0                        # nothing to copy
+    assert h(None, FAKE, 16, None) == _lib.KR_ERR_NULL_POINTER
+    assert h(FAKE, None, 16, None) == _lib.KR_ERR_NULL_POINTER
 
 
 def test_gemm_workspace_entries(lib):

@@ -254,6 +254,31 @@ def test_copy_engine_scatter_overlaps_the_producer(dev, tile, rank):
     assert torch.equal(out, fused.gemm_reduce_scatter_ce_persistent(a.to(dev), b.to(dev), peers=peers.to(dev), rank=rank))
 
 
+def test_copies_on_the_copy_engines(dev):
+    """copy_engine=True: the chunk copies of the all-gather and the band copies of the scatter go
+    through kr_copy_engine_memcpy (SDMA) instead of copy kernels; same bits either way."""
+    from kraken_amd.fused.gemm_reduce_scatter_ce_persistent import copy_engine_scatter, gemm_producer_w_progress
+    W, m, K, N = 4, 256, 512, 384
+    stack = orc.make_stack(W, (m, K), seed0=11)
+    bT = orc.randn_bf16((N, K), 43, 0.05)
+    shards = [stack[r].to(dev) for r in range(W)]
+    status = torch.zeros(1, dtype=torch.int32, device=dev)
+    a_out = torch.full((W * m, K), float("nan"), dtype=BF16, device=dev)
+    ag, c = fused.all_gather_matmul(shards, bT.to(dev).T, a_out=a_out, rank=1, splits_per_rank=2, copy_engine=True,
+                                    status=status)
+    torch.cuda.synchronize()
+    assert status.item() == 0 and torch.equal(ag.cpu(), stack.reshape(W * m, K))
+    assert torch.equal(c, fused.all_gather_matmul(stack.to(dev), bT.to(dev).T)[1])
+    gemm_out = torch.empty(W * m, N, dtype=BF16, device=dev)
+    progress = torch.zeros(W, dtype=torch.int32, device=dev)
+    signal_pad = torch.zeros(W, dtype=torch.int32, device=dev)
+    gemm_producer_w_progress(ag, bT.to(dev).T, gemm_out, progress, signal_pad, {"RANK": 2, "WORLD_SIZE": W})
+    sent = torch.zeros(W, m, N, dtype=BF16, device=dev)
+    copy_engine_scatter(gemm_out, sent, signal_pad, rank=2, status=status, copy_engine=True)
+    torch.cuda.synchronize()
+    assert status.item() == 0 and torch.equal(sent.view(W * m, N), gemm_out)
+
+
 def test_copy_engine_scatter_wait_is_bounded(dev):
     """A flag that never comes: the stream-ordered wait gives up after its limit, records it in
     `status`, and the stream drains."""
