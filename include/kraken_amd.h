@@ -136,7 +136,9 @@ int kr_rmsnorm_bf16(const void* x, const void* w, float eps, int64_t rows, int64
  * tile_pivot: row offset (in rows) by which the order of M tiles is rotated;
  *        changes scheduling only, never the result.
  * Requirements: K % 8 == 0, N % 8 == 0, leading strides % 8 == 0, pointers
- * 16-byte aligned, 0 <= band_row0, band_row0 + band_rows <= M.
+ * 16-byte aligned, 0 <= band_row0, band_row0 + band_rows <= M; row strides up to
+ * about 8 M elements (128 rows of an operand must lie within 2 GiB, else
+ * KR_ERR_LAYOUT).
  * Rounding: the sum is formed in fp32 and rounded once at the store; with a
  * bf16 result, tiles whose peers are added in the epilogue round the product
  * to bf16 before the sum, as gemm_reduce_scatter_fused.py:72 does.

@@ -587,6 +587,13 @@ static int gemm_reduce(const void* A, int64_t lda_m, int64_t lda_k, const void* 
     }
     const bool dtl = big && gemm_dtl_supported(g) &&
                      (g.a_local == nullptr || (int64_t)256 * g.lda_local * 2 < 0x7fffffffLL);
+    // The 128x128 kernel addresses a tile's operand panels with 32-bit byte offsets from the
+    // panel's first row (through a 2 GiB buffer descriptor): row strides beyond that reach are
+    // refused rather than read as zeros.
+    if (!dtl) {
+        const int64_t reach = std::max<int64_t>(std::max(lda_m, ldb), g.a_local != nullptr ? g.lda_local : 0);
+        if ((128 * reach + std::max(K, N)) * 2 >= 0x7fffffffLL) return KR_ERR_LAYOUT;
+    }
     // KRAKEN_AMD_GEMM_PEERS=epilogue keeps the peers' partial sums out of the matrix cores
     // (they are then added in the epilogue, where a non-finite value stays in its element)
     g.peers_on_mfma = 1;

@@ -185,6 +185,15 @@ def test_all_gather_matmul_argument_errors(lib):
     assert g(FAKE + 2, 1, None) == _lib.KR_ERR_ALIGNMENT
 
 
+def test_gemm_row_stride_beyond_the_kernels_reach(lib):
+    # a row stride of 2^24 elements: 128 rows of a tile span 4 GiB, more than the operand descriptors cover
+    f = lib.kr_gemm_reduce_bf16
+    assert f(FAKE, 1 << 24, 1, FAKE, 64, 1, 128, 64, 64, None, 0, 0, None, 0, 128, None, FAKE, 0, 0,
+             None) == _lib.KR_ERR_LAYOUT
+    assert f(FAKE, 64, 1, FAKE, 1, 1 << 24, 128, 64, 64, None, 0, 0, None, 0, 128, None, FAKE, 0, 0,
+             None) == _lib.KR_ERR_LAYOUT
+
+
 def test_gemm_producer_argument_errors(lib):
     f = lib.kr_gemm_producer_bf16
     def args(**kw):
