@@ -199,6 +199,49 @@ def test_ce_persistent_variant(dev, tile):
         torch.testing.assert_close(out.cpu(), want, **TOL)
 
 
+def test_split_k_loop_replays_from_a_graph(dev):
+    """The GEMM entry points enqueue kernels only (the split K loop included: partial products,
+    then the finishing pass): captured once, every replay reproduces the eager result bit for
+    bit, with eager work between the replays."""
+    M, N, K, W = 512, 256, 128, 4
+    a, b, peers = mk(M, N, K, 3, True)
+    bias = orc.randn_bf16((N,), 42, 0.02)
+    ad, bd, pd, biasd = a.to(dev), b.to(dev), peers.to(dev), bias.to(dev)
+    band_peers = torch.stack([orc.randn_bf16((M // W, N), 100 + j) for j in range(W - 1)]).to(dev)
+    c_scratch = torch.empty(M, N, dtype=BF16, device=dev)
+    stack = orc.make_stack(W, (M // W, K)).to(dev)
+    a_few, b_few, _ = mk(128, 384, 1024, 0, False, seed=9)       # 3 tiles: its K loop is split
+    a_few, b_few = a_few.to(dev), b_few.to(dev)
+    assert _lib.load().kr_gemm_workspace_bytes(128, 384, 1024) > 0
+
+    def run():
+        o1 = fused.gemm_one_shot_all_reduce_fused(ad, bd, peers=pd, bias=biasd)
+        o2 = fused.gemm_reduce_scatter(ad, bd, peers=band_peers, rank=1, c_scratch=c_scratch)
+        _, o3 = fused.all_gather_matmul(stack, bd, rank=2)
+        o4 = fused.gemm_one_shot_all_reduce_fused(a_few, b_few)
+        return o1, o2, c_scratch, o3, o4
+
+    eager = [t.clone() for t in run()]
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        run()                                   # the stream's workspace exists before the capture
+        side.synchronize()
+        with torch.cuda.graph(g, stream=side):
+            got = run()
+    for rep in range(3):
+        for t in got:
+            t.zero_()
+        _ = fused.gemm_one_shot_all_reduce_fused(a_few, b_few)   # eager work between the replays
+        torch.cuda.synchronize()
+        g.replay()
+        torch.cuda.synchronize()
+        for e, r in zip(eager, got):
+            assert torch.equal(e, r)
+
+
 def _band_tile_counts(M, N, W, bm):
     rows = M // W
     return [(((r + 1) * rows - 1) // bm - (r * rows) // bm + 1) * -(-N // bm) for r in range(W)]
