@@ -208,7 +208,7 @@ def test_split_k_loop_replays_from_a_graph(dev):
     bias = orc.randn_bf16((N,), 42, 0.02)
     ad, bd, pd, biasd = a.to(dev), b.to(dev), peers.to(dev), bias.to(dev)
     band_peers = torch.stack([orc.randn_bf16((M // W, N), 100 + j) for j in range(W - 1)]).to(dev)
-    c_scratch = torch.empty(M, N, dtype=BF16, device=dev)
+    c_scratch = torch.zeros(M, N, dtype=BF16, device=dev)       # (the own band's rows are never written)
     stack = orc.make_stack(W, (M // W, K)).to(dev)
     a_few, b_few, _ = mk(128, 384, 1024, 0, False, seed=9)       # 3 tiles: its K loop is split
     a_few, b_few = a_few.to(dev), b_few.to(dev)
