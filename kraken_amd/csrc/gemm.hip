@@ -598,6 +598,13 @@ static int gemm_reduce(const void* A, int64_t lda_m, int64_t lda_k, const void* 
     // (they are then added in the epilogue, where a non-finite value stays in its element)
     g.peers_on_mfma = 1;
     if (const char* t = getenv("KRAKEN_AMD_GEMM_PEERS")) g.peers_on_mfma = t[0] == 'e' ? 0 : t[0] == 'f' ? 2 : t[0] == 'l' ? 3 : 1;
+    // MFMA block shape of the 256x256 kernel's k loop: 16x16x32 draws less power per flop than
+    // 32x32x16 and the chip is power-limited (transposed-contiguous B: 4-7 % faster, same bits).
+    // It has no form that adds the peers on the matrix cores, and its transposing reads of a
+    // row-major B run into LDS bank conflicts (25 % slower there), so those calls keep 32x32x16.
+    // KRAKEN_AMD_GEMM_MFMA=16|32 overrides the choice.
+    g.mi16 = b_nt && n_peers == 0;
+    if (const char* t = getenv("KRAKEN_AMD_GEMM_MFMA")) g.mi16 = t[0] == '1';
     const int bm = dtl ? 256 : 128, bn = bm;
     g.tiles_m = (int)((M + bm - 1) / bm);
     g.tiles_n = (int)((N + bn - 1) / bn);

@@ -40,6 +40,7 @@ struct GemmArgs {
     int tail_tiles;
     int group_n;         // column panels per scheduling group (tile_schedule)
     int peers_on_mfma;   // 256x256 kernel: add whole-band tiles' peers through the matrix cores
+    int mi16;            // 256x256 kernel: k loop on 16x16x32 MFMA blocks (peers in the epilogue)
     // producer of the copy-engine reduce-scatter (band_counter == nullptr: off): finished tiles are
     // counted per destination rank, whose band is count_rows rows of C
     uint32_t* band_counter;   // [M / count_rows] tiles finished that touch the band
@@ -156,10 +157,16 @@ __device__ __forceinline__ void tile_schedule(const GemmArgs& g, int pid, int& t
 // the peers and the bias are then added in fp32 in the order own, peer 0, 1, ..., bias.
 // F32 = true (fp32 result: the reference's fused all-reduce keeps fp32 from the accumulator to
 // the output, kraken/fused/gemm_one_shot_all_reduce_fused.py:65-99): the patch holds fp32.
-template <bool F32, int BM, int WTM, int WTN, int TM, int TN, bool EVEN, int EP_WAVE>
+//
+// ACC is either f32x16[TM][TN] (32x32 MFMA blocks: lane l holds row l%32 of a block and the
+// columns 8(v/4) + 4(l/32) + v%4 of register v) or f32x4[2*TM][2*TN] (16x16 blocks: lane l
+// holds row l%16 and the columns 4(l/16) + v); only the copy into the patch knows which.
+template <bool F32, int BM, int WTM, int WTN, int TM, int TN, bool EVEN, int EP_WAVE, class ACC>
 __device__ __forceinline__ void gemm_epilogue_impl(const GemmArgs& g, const int n_peers, const uint16_t* bias,
-                                                   const f32x16 (&acc)[TM][TN], unsigned char* smem,
+                                                   const ACC& acc, unsigned char* smem,
                                                    int m0, int n0, int wm, int wn, int lane, int wave) {
+    constexpr bool MI16 = std::is_same<ACC, f32x4[2 * TM][2 * TN]>::value;
+    static_assert(MI16 || std::is_same<ACC, f32x16[TM][TN]>::value, "unknown accumulator layout");
     // After the barrier above no wave reads the pipeline stages any more, and from here on
     // every wave touches only its own LDS patch, so no further workgroup barrier is needed
     // (LDS requests of one wave are served in order).  Per 32-row slab the accumulators are
@@ -209,10 +216,25 @@ __device__ __forceinline__ void gemm_epilogue_impl(const GemmArgs& g, const int 
     // copy of slab i's accumulators to the patch.  Accumulator registers can only be indexed
     // statically, hence the uniform if-chain inside a rolled slab loop.
     auto copy_slab = [&](int i) __attribute__((always_inline)) {
-        patch_t* row = patch + (lane & 31) * LD + 4 * (lane >> 5);
+        patch_t* row = MI16 ? patch + (lane & 15) * LD + 4 * (lane >> 4) : patch + (lane & 31) * LD + 4 * (lane >> 5);
 #pragma unroll
         for (int ii = 0; ii < TM; ++ii) {
             if (i == ii) {
+                if constexpr (MI16) {
+                    // slab = block rows 2i and 2i+1 (patch rows 0..15 and 16..31), 2*TN column blocks
+#pragma unroll
+                    for (int h = 0; h < 2; ++h)
+#pragma unroll
+                        for (int j = 0; j < 2 * TN; ++j) {
+                            const f32x4& a = acc[2 * ii + h][j];
+                            if constexpr (F32) {
+                                *(f32x4*)(row + h * 16 * LD + j * 16) = a;
+                            } else {
+                                typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+                                *(u32x2*)(row + h * 16 * LD + j * 16) = u32x2{pack_here(a[0], a[1]), pack_here(a[2], a[3])};
+                            }
+                        }
+                } else {
 #pragma unroll
                 for (int j = 0; j < TN; ++j)
 #pragma unroll
@@ -226,6 +248,7 @@ __device__ __forceinline__ void gemm_epilogue_impl(const GemmArgs& g, const int 
                                 u32x2{pack_here(a[4 * q], a[4 * q + 1]), pack_here(a[4 * q + 2], a[4 * q + 3])};
                         }
                     }
+                }
                 // a distinct statement per case: identical case bodies would be merged into one
                 // with a run-time accumulator index, which forces the accumulators into memory
                 asm volatile("; accumulators of slab %0 copied" ::"n"(ii));
@@ -438,12 +461,12 @@ __device__ __forceinline__ void count_finished_tile(const GemmArgs& g, int m0, i
 // n_peers and bias are what is still to be added here (a kernel that has already put the
 // peers or the bias into the accumulators passes 0 / nullptr); g is only read, never copied,
 // so the peer table stays in kernel-argument memory.
-template <int BM, int WTM, int WTN, int TM, int TN, bool EVEN, int EP_WAVE>
+template <int BM, int WTM, int WTN, int TM, int TN, bool EVEN, int EP_WAVE, class ACC>
 __device__ __forceinline__ void gemm_epilogue(const GemmArgs& g, int n_peers, const uint16_t* bias,
-                                              const f32x16 (&acc)[TM][TN], unsigned char* smem,
+                                              const ACC& acc, unsigned char* smem,
                                               int m0, int n0, int wm, int wn, int lane, int wave) {
-    if (g.out_is_fp32) gemm_epilogue_impl<true, BM, WTM, WTN, TM, TN, EVEN, EP_WAVE>(g, n_peers, bias, acc, smem, m0, n0, wm, wn, lane, wave);
-    else gemm_epilogue_impl<false, BM, WTM, WTN, TM, TN, EVEN, EP_WAVE>(g, n_peers, bias, acc, smem, m0, n0, wm, wn, lane, wave);
+    if (g.out_is_fp32) gemm_epilogue_impl<true, BM, WTM, WTN, TM, TN, EVEN, EP_WAVE, ACC>(g, n_peers, bias, acc, smem, m0, n0, wm, wn, lane, wave);
+    else gemm_epilogue_impl<false, BM, WTM, WTN, TM, TN, EVEN, EP_WAVE, ACC>(g, n_peers, bias, acc, smem, m0, n0, wm, wn, lane, wave);
     if (g.band_counter != nullptr) count_finished_tile(g, m0, BM);
 }
 

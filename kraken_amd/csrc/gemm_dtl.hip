@@ -62,8 +62,14 @@ constexpr int kLgkm0 = 0xc07f;   // s_waitcnt lgkmcnt(0) only
 // SPLIT: the workgroup is one of g.k_splits that share a tile of the last partial round: it
 // runs its share of the k-steps and leaves its accumulators in the workspace (no epilogue).
 // RAGGED: M or N is not a multiple of 256 (edge tiles get the bounds-checked epilogue).
-template <bool B_NT, bool PEERS_FIRST, bool SPLIT = false, bool RAGGED = false>
+// MI16: the k loop uses v_mfma_f32_16x16x32_bf16 (8 x 8 blocks of 16 x 16 per wave) instead of
+// 32x32x16 (4 x 4 blocks of 32 x 32): same operand traffic, but the matrix cores draw less power
+// per flop with it (under the power limit, matrix-core-only loops on random operands sustain
+// 2.04 PFLOP/s with 16x16x32 against 1.62 with 32x32x16).  No peers on the matrix cores and no
+// split in this form.
+template <bool B_NT, bool PEERS_FIRST, bool SPLIT = false, bool RAGGED = false, bool MI16 = false>
 __device__ __forceinline__ void gemm_dtl_tile(const GemmArgs& g, unsigned char* smem) {
+    static_assert(!MI16 || !SPLIT, "the split form keeps the 32x32 blocks");
     // Nothing is outstanding at kernel entry; saying so keeps the compiler's own wait-count
     // bookkeeping from carrying the pending loads and stores of the other copy of this code
     // (which never runs in the same workgroup) into this one, where it cannot see the LDS-DMA
@@ -216,6 +222,45 @@ __device__ __forceinline__ void gemm_dtl_tile(const GemmArgs& g, unsigned char* 
         }
     };
 
+    // 16x16x32 blocks: lane -> row (lane & 15) of a 16-row block, 8 k at piece 4*ks2 + (lane >> 4) of
+    // the row's eight (ks2: the two 32-k halves of a stage); blocks are 2 KiB apart.  Row-major B:
+    // the 16-lane group q = lane/16 reads k-rows 8q .. 8q+7 of the half with two transposing reads.
+    uint32_t fa16[2], fb16[2 * TN];
+    bf16x8 af16[2][2 * TM], bfr16[2][2 * TN];
+    if constexpr (MI16) {
+        const int p = lane & 15, gq = lane >> 4;
+        const int sw16 = (p >> 1) & 7;
+#pragma unroll
+        for (int ks2 = 0; ks2 < 2; ++ks2) {
+            fa16[ks2] = (uint32_t)((wm * WTM + p) * 128 + (((4 * ks2 + gq) ^ sw16) << 4));
+            if (B_NT) fb16[ks2] = B_BASE + (uint32_t)((wn * WTN + p) * 128 + (((4 * ks2 + gq) ^ sw16) << 4));
+        }
+        if (!B_NT) {
+#pragma unroll
+            for (int bj = 0; bj < 2 * TN; ++bj) {
+                const int nl = wn * WTN + bj * 16 + 4 * (p & 3);
+                const int kr = 8 * gq + (p >> 2);
+                const int piece = (nl >> 3) ^ (((p >> 2) & 3) << 2);
+                fb16[bj] = B_BASE + (uint32_t)(kr * 512 + piece * 16 + (nl & 7) * 2);
+            }
+        }
+    }
+    auto read_a16 = [&](int buf, int bi, int ks2, uint32_t stage_off) {
+        af16[buf][bi] = *(lds_frag)(size_t)(fa16[ks2] + stage_off + bi * 2048);
+    };
+    auto read_b16 = [&](int buf, int bj, int ks2, uint32_t stage_off) {
+        if (B_NT) {
+            bfr16[buf][bj] = *(lds_frag)(size_t)(fb16[ks2] + stage_off + bj * 2048);
+        } else {
+            const uint32_t a = fb16[bj] + stage_off + ks2 * 16384;
+            const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_tr)(size_t)a);
+            const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_tr)(size_t)(a + 2048));
+            typedef short s16x8 __attribute__((ext_vector_type(8)));
+            const s16x8 v = {lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+            bfr16[buf][bj] = __builtin_bit_cast(bf16x8, v);
+        }
+    };
+
     // The accumulators start at the bias instead of zero when the whole tile lies in the reduce
     // band and nothing is left for the epilogue to add in bf16 (no peers, or peers added on the
     // matrix cores): product, partial sums and bias are then summed in fp32 and rounded once,
@@ -225,7 +270,7 @@ __device__ __forceinline__ void gemm_dtl_tile(const GemmArgs& g, unsigned char* 
     const int band_lo = g.band_row0;
     const bool full_tile = !RAGGED || (m0 + BM <= g.M && n0 + BN <= g.N);
     const bool tile_in_band = full_tile && m0 >= band_lo && m0 + BM <= band_lo + g.band_rows;
-    const bool mfma_peers = !SPLIT && g.peers_on_mfma && g.n_peers > 0 && tile_in_band;
+    const bool mfma_peers = !SPLIT && !MI16 && g.peers_on_mfma && g.n_peers > 0 && tile_in_band;
     const bool bias_in_acc = !SPLIT && g.bias != nullptr && tile_in_band && (g.n_peers == 0 || mfma_peers);
     f32x16 acc[TM][TN];
     {
@@ -252,6 +297,27 @@ __device__ __forceinline__ void gemm_dtl_tile(const GemmArgs& g, unsigned char* 
         for (int i = 0; i < TM; ++i)
 #pragma unroll
             for (int j = 0; j < TN; ++j) acc[i][j] = init[j];
+    }
+
+    // the same for the 16x16 blocks: a lane holds row lane%16 and the columns 16j + 4(lane/16) .. +3
+    f32x4 acc16[2 * TM][2 * TN];
+    if constexpr (MI16) {
+        f32x4 init16[2 * TN];
+#pragma unroll
+        for (int j = 0; j < 2 * TN; ++j) init16[j] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+        if (bias_in_acc) {
+            typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+            const uint16_t* bp = g.bias + n0 + wn * WTN + 4 * (lane >> 4);
+#pragma unroll
+            for (int j = 0; j < 2 * TN; ++j) {
+                const u32x2 b4 = *(const u32x2*)(bp + j * 16);
+                init16[j] = f32x4{bf16_lo(b4.x), bf16_hi(b4.x), bf16_lo(b4.y), bf16_hi(b4.y)};
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < 2 * TM; ++i)
+#pragma unroll
+            for (int j = 0; j < 2 * TN; ++j) acc16[i][j] = init16[j];
     }
 
 #define KR_SCHED_FENCE() __builtin_amdgcn_sched_barrier(0)
@@ -342,10 +408,17 @@ __device__ __forceinline__ void gemm_dtl_tile(const GemmArgs& g, unsigned char* 
     // phases: with the live ranges cut here the register allocator keeps the accumulators
     // where the MFMAs left them instead of moving them to VGPRs and memory for the next phase.
     auto pin_accumulators = [&]() __attribute__((always_inline)) {
+        if constexpr (MI16) {
 #pragma unroll
-        for (int i = 0; i < TM; ++i)
+            for (int i = 0; i < 2 * TM; ++i)
 #pragma unroll
-            for (int j = 0; j < TN; ++j) asm volatile("" : "+a"(acc[i][j]));
+                for (int j = 0; j < 2 * TN; ++j) asm volatile("" : "+a"(acc16[i][j]));
+        } else {
+#pragma unroll
+            for (int i = 0; i < TM; ++i)
+#pragma unroll
+                for (int j = 0; j < TN; ++j) asm volatile("" : "+a"(acc[i][j]));
+        }
     };
     if (PEERS_FIRST && mfma_peers) peer_phase();
     pin_accumulators();
@@ -365,10 +438,17 @@ __device__ __forceinline__ void gemm_dtl_tile(const GemmArgs& g, unsigned char* 
     __builtin_amdgcn_s_waitcnt(vmcnt_imm(kEarly));
     __builtin_amdgcn_s_barrier();
     KR_SCHED_FENCE();
+    if constexpr (MI16) {
 #pragma unroll
-    for (int i = 0; i < TM; ++i) read_a(0, i, 0, 0);
+        for (int i = 0; i < 2 * TM; ++i) read_a16(0, i, 0, 0);
 #pragma unroll
-    for (int j = 0; j < TN; ++j) read_b(0, j, 0, 0);
+        for (int j = 0; j < 2 * TN; ++j) read_b16(0, j, 0, 0);
+    } else {
+#pragma unroll
+        for (int i = 0; i < TM; ++i) read_a(0, i, 0, 0);
+#pragma unroll
+        for (int j = 0; j < TN; ++j) read_b(0, j, 0, 0);
+    }
 
     // ---- main loop ---------------------------------------------------------------------------
     // k-step t (64 k): 4 sub-steps of 16 MFMAs on alternating fragment buffers; sub-step ks
@@ -412,17 +492,66 @@ __device__ __forceinline__ void gemm_dtl_tile(const GemmArgs& g, unsigned char* 
             }
         }
     };
+    // The same k-step on 16x16x32 blocks: two sub-steps of 64 MFMAs (32 k each) on alternating
+    // fragment buffers.  The fragments of sub-step 1 are read during sub-step 0 (one read every
+    // second MFMA); the first row of MFMAs of sub-step 1 consumes the last of them, so behind
+    // MFMA 7 every LDS read of the stage has returned: wait for the loads of step t+1, barrier,
+    // then the first fragments of step t+1 and the first loads of step t+2.
+    constexpr int NM16 = 4 * TM * TN;
+    auto k_step16 = [&](int t, auto stage_c) __attribute__((always_inline)) {
+        const uint32_t stage_cur = stage_c;
+        const uint32_t stage_nxt = stage_cur ^ 1u;
+        const uint32_t st_cur = stage_cur * A_ST, st_nxt = stage_nxt * A_ST;
+#pragma unroll
+        for (int ks2 = 0; ks2 < 2; ++ks2) {
+            const int cur = ks2, nxt = cur ^ 1;
+#pragma unroll
+            for (int s = 0; s < NM16; ++s) {
+                const int i = s / (2 * TN), j = s % (2 * TN);
+                acc16[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(bfr16[cur][j], af16[cur][i], acc16[i][j], 0, 0, 0);
+                if (ks2 == 0) {
+                    if (s % 2 == 0 && s < 4 * TM) read_a16(nxt, s / 2, 1, st_cur);
+                    else if (s % 2 == 0 && s < 4 * TM + 4 * TN) read_b16(nxt, (s - 4 * TM) / 2, 1, st_cur);
+                    // the later loads of step t+1
+                    if (s % 4 == 1 && s / 4 < LOADS_PER_TILE - kEarly) issue_load(t + 1, stage_nxt, kEarly + s / 4);
+                } else {
+                    if (s == 2 * TN - 1) {
+                        KR_SCHED_FENCE();
+                        __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));
+                        __builtin_amdgcn_s_barrier();
+                    }
+                    // first fragments of k-step t+1
+                    if (s >= 2 * TN && s % 2 == 0 && s < 2 * TN + 4 * TM) read_a16(nxt, (s - 2 * TN) / 2, 0, st_nxt);
+                    else if (s >= 2 * TN + 4 * TM && s % 2 == 0 && s < 2 * TN + 4 * TM + 4 * TN)
+                        read_b16(nxt, (s - 2 * TN - 4 * TM) / 2, 0, st_nxt);
+                    // the first loads of step t+2, into the stage just vacated
+                    if (s > 2 * TN && s % 4 == 1 && (s - 2 * TN - 1) / 4 < kEarly) issue_load(t + 2, stage_cur, (s - 2 * TN - 1) / 4);
+                }
+                KR_SCHED_FENCE();
+            }
+        }
+    };
     // Main part: one trip = two k-steps, so every LDS stage offset is a compile-time constant
     // (immediate offsets on the fragment reads) and the loop branch is taken once per 128 MFMAs;
     // an odd last step follows.
     int t = 0;
+    if constexpr (MI16) {
 #pragma nounroll
-    for (; t + 2 <= kt_total; t += 2) {
-        k_step(t, std::integral_constant<uint32_t, 0>{});
-        k_step(t + 1, std::integral_constant<uint32_t, 1>{});
+        for (; t + 2 <= kt_total; t += 2) {
+            k_step16(t, std::integral_constant<uint32_t, 0>{});
+            k_step16(t + 1, std::integral_constant<uint32_t, 1>{});
+        }
+        pin_accumulators();
+        if (t < kt_total) k_step16(t, std::integral_constant<uint32_t, 0>{});
+    } else {
+#pragma nounroll
+        for (; t + 2 <= kt_total; t += 2) {
+            k_step(t, std::integral_constant<uint32_t, 0>{});
+            k_step(t + 1, std::integral_constant<uint32_t, 1>{});
+        }
+        pin_accumulators();
+        if (t < kt_total) k_step(t, std::integral_constant<uint32_t, 0>{});
     }
-    pin_accumulators();
-    if (t < kt_total) k_step(t, std::integral_constant<uint32_t, 0>{});
     // drain the tail's surplus loads before the LDS is reused
     __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));
     __syncthreads();
@@ -446,7 +575,14 @@ __device__ __forceinline__ void gemm_dtl_tile(const GemmArgs& g, unsigned char* 
     if (!PEERS_FIRST && mfma_peers) peer_phase();
     pin_accumulators();
     // peers and bias that are already in the accumulators are not added again
-    if (full_tile) {
+    if constexpr (MI16) {
+        if (full_tile) {
+            gemm_epilogue<BM, WTM, WTN, TM, TN, true, EP_WAVE>(g, g.n_peers, bias_in_acc ? nullptr : g.bias, acc16, smem, m0, n0,
+                                                               wm, wn, lane, wave);
+        } else if constexpr (RAGGED) {
+            gemm_epilogue<BM, WTM, WTN, TM, TN, false, EP_WAVE>(g, g.n_peers, g.bias, acc16, smem, m0, n0, wm, wn, lane, wave);
+        }
+    } else if (full_tile) {
         gemm_epilogue<BM, WTM, WTN, TM, TN, true, EP_WAVE>(g, mfma_peers ? 0 : g.n_peers, bias_in_acc ? nullptr : g.bias,
                                                            acc, smem, m0, n0, wm, wn, lane, wave);
     } else if constexpr (RAGGED) {   // edge tile: every access checked against M and N
@@ -463,6 +599,13 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_dtl_kernel(const GemmArgs g)
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];   // starts at LDS address 0
     if (g.peers_on_mfma && g.n_peers > 0 && (g.peers_on_mfma == 1 ? ((blockIdx.x >> 3) & 1) : g.peers_on_mfma == 2)) gemm_dtl_tile<B_NT, true, false, RAGGED>(g, smem);
     else gemm_dtl_tile<B_NT, false, false, RAGGED>(g, smem);
+}
+
+// The k loop on 16x16x32 blocks (peers, if any, are added in the epilogue).
+template <bool B_NT, bool RAGGED>
+__global__ __launch_bounds__(WM* WN * 64) void gemm_dtl16_kernel(const GemmArgs g) {
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+    gemm_dtl_tile<B_NT, false, false, RAGGED, true>(g, smem);
 }
 
 }  // namespace
@@ -525,10 +668,22 @@ hipError_t launch_gemm_dtl(const GemmArgs& g, bool b_nt, hipStream_t st, void* w
     const bool ragged = g.M % BM != 0 || g.N % BN != 0;
     const void* kfn = b_nt ? (ragged ? (const void*)gemm_dtl_kernel<true, true> : (const void*)gemm_dtl_kernel<true, false>)
                            : (ragged ? (const void*)gemm_dtl_kernel<false, true> : (const void*)gemm_dtl_kernel<false, false>);
-    static std::atomic<uint64_t> opted[4];
-    if (hipError_t e = lds_opt_in(kfn, LDS_BYTES, opted[(b_nt ? 2 : 0) + (ragged ? 1 : 0)]); e != hipSuccess) return e;
+    if (g.mi16)
+        kfn = b_nt ? (ragged ? (const void*)gemm_dtl16_kernel<true, true> : (const void*)gemm_dtl16_kernel<true, false>)
+                   : (ragged ? (const void*)gemm_dtl16_kernel<false, true> : (const void*)gemm_dtl16_kernel<false, false>);
+    static std::atomic<uint64_t> opted[8];
+    if (hipError_t e = lds_opt_in(kfn, LDS_BYTES, opted[(g.mi16 ? 4 : 0) + (b_nt ? 2 : 0) + (ragged ? 1 : 0)]); e != hipSuccess)
+        return e;
     if (grid.x == 0) {
         // every tile belongs to the split partial round
+    } else if (g.mi16) {
+        if (b_nt) {
+            if (ragged) hipLaunchKernelGGL((gemm_dtl16_kernel<true, true>), grid, block, LDS_BYTES, st, g);
+            else hipLaunchKernelGGL((gemm_dtl16_kernel<true, false>), grid, block, LDS_BYTES, st, g);
+        } else {
+            if (ragged) hipLaunchKernelGGL((gemm_dtl16_kernel<false, true>), grid, block, LDS_BYTES, st, g);
+            else hipLaunchKernelGGL((gemm_dtl16_kernel<false, false>), grid, block, LDS_BYTES, st, g);
+        }
     } else if (b_nt) {
         if (ragged) hipLaunchKernelGGL((gemm_dtl_kernel<true, true>), grid, block, LDS_BYTES, st, g);
         else hipLaunchKernelGGL((gemm_dtl_kernel<true, false>), grid, block, LDS_BYTES, st, g);
