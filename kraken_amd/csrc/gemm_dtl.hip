@@ -108,7 +108,7 @@ __device__ __forceinline__ void gemm_dtl_tile(const GemmArgs& g, unsigned char* 
     // part (chunk row, k) goes to the scalar offset.
     const int dma_sw = (4 * (wave & 1) + (lane >> 4)) & 7;
     const uint32_t a_voff_lane = (uint32_t)(((int64_t)(lane >> 3) * lda + (((lane & 7) ^ dma_sw) << 3)) * 2);
-    uint32_t b_voff_lane;
+    uint32_t b_voff_lane, b_voff_odd = 0;
     if (B_NT) {
         b_voff_lane = (uint32_t)(((int64_t)(lane >> 3) * g.ldb + (((lane & 7) ^ dma_sw) << 3)) * 2);
     } else {
@@ -116,6 +116,10 @@ __device__ __forceinline__ void gemm_dtl_tile(const GemmArgs& g, unsigned char* 
         // slot ^ 4*(k & 3); k & 3 = 2*(chunk & 1) + l/32 and chunk & 1 == wave & 1
         const int kq = ((wave & 1) << 1) | (lane >> 5);
         b_voff_lane = (uint32_t)(((int64_t)(lane >> 5) * g.ldb + (((lane & 31) ^ (kq << 2)) << 3)) * 2);
+        // 16x16x32 blocks: all four 16-lane groups of a transposing read want the same 16 columns,
+        // of k-rows 8 apart; a further XOR with 2*((k >> 3) & 1) puts groups 0/1 (2/3) on different
+        // banks.  (k >> 3) & 1 = chunk parity of the load's index, a second offset for the odd ones.
+        if (MI16) b_voff_odd = (uint32_t)(((int64_t)(lane >> 5) * g.ldb + (((lane & 31) ^ (kq << 2) ^ 2) << 3)) * 2);
     }
     // Buffer resource descriptor: 48-bit base, stride 0 (raw), 2^31-1 bytes, 32-bit data format.
     typedef int i32x4 __attribute__((ext_vector_type(4)));
@@ -160,7 +164,8 @@ __device__ __forceinline__ void gemm_dtl_tile(const GemmArgs& g, unsigned char* 
         const bool live = t < kt_total;
         const int tt = min(t, kt_total - 1);
         const int k0 = tt * BKD;
-        const uint32_t a_voff = live ? a_voff_lane : 0u, b_voff = live ? b_voff_lane : 0u;
+        const uint32_t a_voff = live ? a_voff_lane : 0u;
+        const uint32_t b_voff = !live ? 0u : (MI16 && !B_NT && ((q % LOADS_A) & 1)) ? b_voff_odd : b_voff_lane;
         const int ch = wave + 4 * (q % LOADS_A);
         if (q < LOADS_A) {
             lds_dma_b128(a_rsrc, stage * A_ST + ch * 1024, a_voff, (int)(((int64_t)8 * ch * lda + k0) * 2));
@@ -240,7 +245,7 @@ __device__ __forceinline__ void gemm_dtl_tile(const GemmArgs& g, unsigned char* 
             for (int bj = 0; bj < 2 * TN; ++bj) {
                 const int nl = wn * WTN + bj * 16 + 4 * (p & 3);
                 const int kr = 8 * gq + (p >> 2);
-                const int piece = (nl >> 3) ^ (((p >> 2) & 3) << 2);
+                const int piece = (nl >> 3) ^ (((p >> 2) & 3) << 2) ^ ((gq & 1) << 1);
                 fb16[bj] = B_BASE + (uint32_t)(kr * 512 + piece * 16 + (nl & 7) * 2);
             }
         }
@@ -508,7 +513,16 @@ __device__ __forceinline__ void gemm_dtl_tile(const GemmArgs& g, unsigned char* 
 #pragma unroll
             for (int s = 0; s < NM16; ++s) {
                 const int i = s / (2 * TN), j = s % (2 * TN);
-                acc16[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(bfr16[cur][j], af16[cur][i], acc16[i][j], 0, 0, 0);
+                if constexpr (B_NT) {
+                    acc16[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(bfr16[cur][j], af16[cur][i], acc16[i][j], 0, 0, 0);
+                } else {
+                    // (written out with the accumulator tied to the AGPRs it lives in: left to the
+                    // register allocator, the row-major-B form moves accumulators through VGPRs
+                    // around every MFMA)
+                    asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0"
+                                 : "+a"(acc16[i][j])
+                                 : "v"(bfr16[cur][j]), "v"(af16[cur][i]));
+                }
                 if (ks2 == 0) {
                     if (s % 2 == 0 && s < 4 * TM) read_a16(nxt, s / 2, 1, st_cur);
                     else if (s % 2 == 0 && s < 4 * TM + 4 * TN) read_b16(nxt, (s - 4 * TM) / 2, 1, st_cur);
