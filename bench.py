@@ -253,7 +253,7 @@ class GemmReduceScatter(Workload):
         return orc.gemm_reduce_scatter(self.ha, self.hb, self.hp, self.rank, W)
 
     def describe(self):
-        return {"M": self.M, "N": self.N, "K": self.K, "peers": [7, 1024, self.N], "kernel": "gemm_dtl_kernel"}
+        return {"M": self.M, "N": self.N, "K": self.K, "peers": [7, 1024, self.N], "kernel": "gemm_dtl16_kernel"}
 
 
 class GemmAllReduce(Workload):
@@ -346,7 +346,7 @@ class AllGatherMatmul(Workload):
         return orc.all_gather_matmul(self.hs, self.hbT.T)
 
     def describe(self):
-        return {"W": W, "m": self.m, "K": self.K, "N": self.N, "b_layout": "b.T contiguous", "kernel": "gemm_dtl_kernel"}
+        return {"W": W, "m": self.m, "K": self.K, "N": self.N, "b_layout": "b.T contiguous", "kernel": "gemm_dtl16_kernel"}
 
 
 def make_workloads():

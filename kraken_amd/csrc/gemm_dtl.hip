@@ -65,11 +65,10 @@ constexpr int kLgkm0 = 0xc07f;   // s_waitcnt lgkmcnt(0) only
 // MI16: the k loop uses v_mfma_f32_16x16x32_bf16 (8 x 8 blocks of 16 x 16 per wave) instead of
 // 32x32x16 (4 x 4 blocks of 32 x 32): same operand traffic, but the matrix cores draw less power
 // per flop with it (under the power limit, matrix-core-only loops on random operands sustain
-// 2.04 PFLOP/s with 16x16x32 against 1.62 with 32x32x16).  No peers on the matrix cores and no
-// split in this form.
+// 2.04 PFLOP/s with 16x16x32 against 1.62 with 32x32x16).  No peers on the matrix cores in this
+// form.
 template <bool B_NT, bool PEERS_FIRST, bool SPLIT = false, bool RAGGED = false, bool MI16 = false>
 __device__ __forceinline__ void gemm_dtl_tile(const GemmArgs& g, unsigned char* smem) {
-    static_assert(!MI16 || !SPLIT, "the split form keeps the 32x32 blocks");
     // Nothing is outstanding at kernel entry; saying so keeps the compiler's own wait-count
     // bookkeeping from carrying the pending loads and stores of the other copy of this code
     // (which never runs in the same workgroup) into this one, where it cannot see the LDS-DMA
@@ -575,6 +574,14 @@ __device__ __forceinline__ void gemm_dtl_tile(const GemmArgs& g, unsigned char* 
         // accumulators to the workspace in register order: quad q = (i, j, v/4) of thread tid at
         // [tail tile][split][q][tid], so that a wave's store is 1 KiB of consecutive addresses
         f32x4* part = (f32x4*)g.out + ((int64_t)tail_index * g.k_splits + split) * (TM * TN * 4 * WM * WN * 64) + tid;
+        if constexpr (MI16) {   // quad q = block (i, j) of the 8 x 8
+#pragma unroll
+            for (int i = 0; i < 2 * TM; ++i)
+#pragma unroll
+                for (int j = 0; j < 2 * TN; ++j)
+                    __builtin_nontemporal_store(acc16[i][j], part + (i * 2 * TN + j) * (WM * WN * 64));
+            return;
+        }
 #pragma unroll
         for (int i = 0; i < TM; ++i)
 #pragma unroll
@@ -626,10 +633,10 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_dtl16_kernel(const GemmArgs 
 
 // Second launch of a call with a split tail: g.k_splits workgroups per tile of the last partial
 // round (g.out = workspace).
-template <bool B_NT>
+template <bool B_NT, bool MI16>
 __global__ __launch_bounds__(WM* WN * 64) void gemm_dtl_split_kernel(const GemmArgs g) {
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
-    gemm_dtl_tile<B_NT, false, true>(g, smem);
+    gemm_dtl_tile<B_NT, false, true, false, MI16>(g, smem);
 }
 
 // Third launch: sums the parts of every tail tile in the order 0..S-1 and applies the epilogue
@@ -649,9 +656,15 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_dtl_tail_finish_kernel(const
     }
     int tile_m, tile_n;
     tile_schedule(g, schedule_position(g, u, g.tiles_m * g.tiles_n - g.tail_tiles), tile_m, tile_n);
-    const int i = q / (TN * 4), j = (q / 4) % TN, v4 = q % 4;
-    const int m = tile_m * BM + (wave / WN) * WTM + i * 32 + (lane & 31);
-    const int n = tile_n * BN + (wave % WN) * WTN + j * 32 + 8 * v4 + 4 * (lane >> 5);
+    int m, n;
+    if (g.mi16) {   // 16x16 blocks: quad q = block (q / 16, q % 16); row lane%16, columns 4(lane/16) .. +3
+        m = tile_m * BM + (wave / WN) * WTM + (q / (2 * TN)) * 16 + (lane & 15);
+        n = tile_n * BN + (wave % WN) * WTN + (q % (2 * TN)) * 16 + 4 * (lane >> 4);
+    } else {
+        const int i = q / (TN * 4), j = (q / 4) % TN, v4 = q % 4;
+        m = tile_m * BM + (wave / WN) * WTM + i * 32 + (lane & 31);
+        n = tile_n * BN + (wave % WN) * WTN + j * 32 + 8 * v4 + 4 * (lane >> 5);
+    }
     typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
     const int mb = m - g.band_row0;
     if (mb < 0 || mb >= g.band_rows) {
@@ -708,18 +721,22 @@ hipError_t launch_gemm_dtl(const GemmArgs& g, bool b_nt, hipStream_t st, void* w
     if (g.tail_tiles > 0) {
         // the tiles of the last partial round: k_splits workgroups each, parts to the workspace,
         // then the sum and the epilogue
-        static std::atomic<uint64_t> split_opted[2];
-        const void* sfn = b_nt ? (const void*)gemm_dtl_split_kernel<true> : (const void*)gemm_dtl_split_kernel<false>;
-        if (hipError_t e2 = lds_opt_in(sfn, LDS_BYTES, split_opted[b_nt]); e2 != hipSuccess) return e2;
+        static std::atomic<uint64_t> split_opted[4];
+        const void* sfn = g.mi16 ? (b_nt ? (const void*)gemm_dtl_split_kernel<true, true> : (const void*)gemm_dtl_split_kernel<false, true>)
+                                 : (b_nt ? (const void*)gemm_dtl_split_kernel<true, false> : (const void*)gemm_dtl_split_kernel<false, false>);
+        if (hipError_t e2 = lds_opt_in(sfn, LDS_BYTES, split_opted[(g.mi16 ? 2 : 0) + (b_nt ? 1 : 0)]); e2 != hipSuccess) return e2;
         hipError_t e = hipGetLastError();
         if (e != hipSuccess) return e;
         GemmArgs gs = g;
         gs.out = workspace;
         const dim3 sgrid((unsigned)(g.tail_tiles * g.k_splits));
-        if (b_nt)
-            hipLaunchKernelGGL(gemm_dtl_split_kernel<true>, sgrid, block, LDS_BYTES, st, gs);
-        else
-            hipLaunchKernelGGL(gemm_dtl_split_kernel<false>, sgrid, block, LDS_BYTES, st, gs);
+        if (g.mi16) {
+            if (b_nt) hipLaunchKernelGGL((gemm_dtl_split_kernel<true, true>), sgrid, block, LDS_BYTES, st, gs);
+            else hipLaunchKernelGGL((gemm_dtl_split_kernel<false, true>), sgrid, block, LDS_BYTES, st, gs);
+        } else {
+            if (b_nt) hipLaunchKernelGGL((gemm_dtl_split_kernel<true, false>), sgrid, block, LDS_BYTES, st, gs);
+            else hipLaunchKernelGGL((gemm_dtl_split_kernel<false, false>), sgrid, block, LDS_BYTES, st, gs);
+        }
         e = hipGetLastError();
         if (e != hipSuccess) return e;
         hipLaunchKernelGGL(gemm_dtl_tail_finish_kernel, dim3((unsigned)(g.tail_tiles * TM * TN * 4)), block, 0, st, g,
