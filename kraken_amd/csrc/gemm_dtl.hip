@@ -433,7 +433,10 @@ __device__ __forceinline__ void gemm_dtl_tile(const GemmArgs& g, unsigned char* 
     // 1 of step t-1 -- every second MFMA.  One per MFMA from four waves is twice what the CU's
     // address unit takes (the waves then stall at issue); spreading them evenly over the whole
     // step leaves the last ones too little time before the barrier that needs them.
-    constexpr int kEarly = 6;
+    // (16x16x32 form: its MFMAs are half as long, so a load issued during the step that needs it
+    // has half as many MFMAs to hide behind; there all loads of step t+2 go out behind the barrier
+    // of step t, one per three MFMAs)
+    constexpr int kEarly = MI16 ? LOADS_PER_TILE : 6;
     static_assert(NSTAGE == 2 && LOADS_PER_TILE == 16, "load schedule below: 6 + 8 + 2 loads");
 #pragma unroll
     for (int q = 0; q < LOADS_PER_TILE; ++q) issue_load(0, 0, q);
@@ -497,11 +500,17 @@ __device__ __forceinline__ void gemm_dtl_tile(const GemmArgs& g, unsigned char* 
         }
     };
     // The same k-step on 16x16x32 blocks: two sub-steps of 64 MFMAs (32 k each) on alternating
-    // fragment buffers.  The fragments of sub-step 1 are read during sub-step 0 (one read every
-    // second MFMA); the first row of MFMAs of sub-step 1 consumes the last of them, so behind
-    // MFMA 7 every LDS read of the stage has returned: wait for the loads of step t+1, barrier,
-    // then the first fragments of step t+1 and the first loads of step t+2.
+    // fragment buffers.  An MFMA lasts 16 cycles here, room for about three other instructions,
+    // so fragment reads and loads are spread one per slot: during sub-step 0 the 16 fragments of
+    // sub-step 1 (every fourth MFMA; B blocks first, then the A blocks in the order the rows of
+    // MFMAs need them).  Behind MFMA 7 of sub-step 1 all of them have long returned: wait for the
+    // loads of step t+1, barrier; then, every third MFMA each, the first fragments of step t+1 and
+    // all 16 loads of step t+2 into the stage just vacated.
     constexpr int NM16 = 4 * TM * TN;
+    auto read_frag16 = [&](int buf, int r, int ks2, uint32_t stage_off) __attribute__((always_inline)) {
+        if (r < 2 * TN) read_b16(buf, r, ks2, stage_off);
+        else read_a16(buf, r - 2 * TN, ks2, stage_off);
+    };
     auto k_step16 = [&](int t, auto stage_c) __attribute__((always_inline)) {
         const uint32_t stage_cur = stage_c;
         const uint32_t stage_nxt = stage_cur ^ 1u;
@@ -512,33 +521,26 @@ __device__ __forceinline__ void gemm_dtl_tile(const GemmArgs& g, unsigned char* 
 #pragma unroll
             for (int s = 0; s < NM16; ++s) {
                 const int i = s / (2 * TN), j = s % (2 * TN);
-                if constexpr (B_NT) {
-                    acc16[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(bfr16[cur][j], af16[cur][i], acc16[i][j], 0, 0, 0);
-                } else {
-                    // (written out with the accumulator tied to the AGPRs it lives in: left to the
-                    // register allocator, the row-major-B form moves accumulators through VGPRs
-                    // around every MFMA)
-                    asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0"
-                                 : "+a"(acc16[i][j])
-                                 : "v"(bfr16[cur][j]), "v"(af16[cur][i]));
-                }
+                // (written out with the accumulator tied to the AGPRs it lives in: given the
+                // builtin, the register allocator moves accumulators through VGPRs and other
+                // AGPRs around the MFMAs, a copy or two per MFMA)
+                asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0"
+                             : "+a"(acc16[i][j])
+                             : "v"(bfr16[cur][j]), "v"(af16[cur][i]));
                 if (ks2 == 0) {
-                    if (s % 2 == 0 && s < 4 * TM) read_a16(nxt, s / 2, 1, st_cur);
-                    else if (s % 2 == 0 && s < 4 * TM + 4 * TN) read_b16(nxt, (s - 4 * TM) / 2, 1, st_cur);
-                    // the later loads of step t+1
-                    if (s % 4 == 1 && s / 4 < LOADS_PER_TILE - kEarly) issue_load(t + 1, stage_nxt, kEarly + s / 4);
+                    if (s % 4 == 0) read_frag16(nxt, s / 4, 1, st_cur);
                 } else {
-                    if (s == 2 * TN - 1) {
+                    constexpr int kBar = 2 * TN - 1;   // last MFMA of the first row
+                    if (s == kBar) {
                         KR_SCHED_FENCE();
+                        __builtin_amdgcn_s_waitcnt(kLgkm0);
                         __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));
                         __builtin_amdgcn_s_barrier();
                     }
-                    // first fragments of k-step t+1
-                    if (s >= 2 * TN && s % 2 == 0 && s < 2 * TN + 4 * TM) read_a16(nxt, (s - 2 * TN) / 2, 0, st_nxt);
-                    else if (s >= 2 * TN + 4 * TM && s % 2 == 0 && s < 2 * TN + 4 * TM + 4 * TN)
-                        read_b16(nxt, (s - 2 * TN - 4 * TM) / 2, 0, st_nxt);
-                    // the first loads of step t+2, into the stage just vacated
-                    if (s > 2 * TN && s % 4 == 1 && (s - 2 * TN - 1) / 4 < kEarly) issue_load(t + 2, stage_cur, (s - 2 * TN - 1) / 4);
+                    if (s > kBar && (s - kBar - 1) % 3 == 0 && (s - kBar - 1) / 3 < 4 * (TM + TN) / 2)
+                        read_frag16(nxt, (s - kBar - 1) / 3, 0, st_nxt);
+                    if (s > kBar && (s - kBar - 1) % 3 == 1 && (s - kBar - 1) / 3 < LOADS_PER_TILE)
+                        issue_load(t + 2, stage_cur, (s - kBar - 1) / 3);
                 }
                 KR_SCHED_FENCE();
             }
