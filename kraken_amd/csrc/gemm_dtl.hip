@@ -434,9 +434,10 @@ __device__ __forceinline__ void gemm_dtl_tile(const GemmArgs& g, unsigned char* 
     // address unit takes (the waves then stall at issue); spreading them evenly over the whole
     // step leaves the last ones too little time before the barrier that needs them.
     // (16x16x32 form: its MFMAs are half as long, so a load issued during the step that needs it
-    // has half as many MFMAs to hide behind; there all loads of step t+2 go out behind the barrier
-    // of step t, one per three MFMAs)
-    constexpr int kEarly = MI16 ? LOADS_PER_TILE : 6;
+    // has half as many MFMAs to hide behind; there 14 loads of step t+2 go out behind the barrier
+    // of step t, one per four MFMAs -- 64 cycles apart, as above -- and the last two at the start
+    // of step t+1)
+    constexpr int kEarly = MI16 ? 14 : 6;
     static_assert(NSTAGE == 2 && LOADS_PER_TILE == 16, "load schedule below: 6 + 8 + 2 loads");
 #pragma unroll
     for (int q = 0; q < LOADS_PER_TILE; ++q) issue_load(0, 0, q);
@@ -504,8 +505,9 @@ __device__ __forceinline__ void gemm_dtl_tile(const GemmArgs& g, unsigned char* 
     // so fragment reads and loads are spread one per slot: during sub-step 0 the 16 fragments of
     // sub-step 1 (every fourth MFMA; B blocks first, then the A blocks in the order the rows of
     // MFMAs need them).  Behind MFMA 7 of sub-step 1 all of them have long returned: wait for the
-    // loads of step t+1, barrier; then, every third MFMA each, the first fragments of step t+1 and
-    // all 16 loads of step t+2 into the stage just vacated.
+    // loads of step t+1, barrier; then, in slots of their own, the first fragments of step t+1 and
+    // 14 of the 16 loads of step t+2 into the stage just vacated (the last two follow at the start
+    // of the next step).
     constexpr int NM16 = 4 * TM * TN;
     auto read_frag16 = [&](int buf, int r, int ks2, uint32_t stage_off) __attribute__((always_inline)) {
         if (r < 2 * TN) read_b16(buf, r, ks2, stage_off);
@@ -529,6 +531,8 @@ __device__ __forceinline__ void gemm_dtl_tile(const GemmArgs& g, unsigned char* 
                              : "v"(bfr16[cur][j]), "v"(af16[cur][i]));
                 if (ks2 == 0) {
                     if (s % 4 == 0) read_frag16(nxt, s / 4, 1, st_cur);
+                    // the last loads of step t+1
+                    if (s % 4 == 1 && s / 4 < LOADS_PER_TILE - kEarly) issue_load(t + 1, stage_nxt, kEarly + s / 4);
                 } else {
                     constexpr int kBar = 2 * TN - 1;   // last MFMA of the first row
                     if (s == kBar) {
@@ -537,10 +541,12 @@ __device__ __forceinline__ void gemm_dtl_tile(const GemmArgs& g, unsigned char* 
                         __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));
                         __builtin_amdgcn_s_barrier();
                     }
-                    if (s > kBar && (s - kBar - 1) % 3 == 0 && (s - kBar - 1) / 3 < 4 * (TM + TN) / 2)
-                        read_frag16(nxt, (s - kBar - 1) / 3, 0, st_nxt);
-                    if (s > kBar && (s - kBar - 1) % 3 == 1 && (s - kBar - 1) / 3 < LOADS_PER_TILE)
-                        issue_load(t + 2, stage_cur, (s - kBar - 1) / 3);
+                    // (slots 8, 11, 12, then every fourth from 15: none shared with a load)
+                    const int rd = s == kBar + 1 ? 0 : s == kBar + 4 ? 1 : s == kBar + 5 ? 2
+                                   : (s >= kBar + 8 && (s - kBar - 8) % 4 == 0) ? 3 + (s - kBar - 8) / 4 : -1;
+                    if (rd >= 0 && rd < 2 * (TM + TN)) read_frag16(nxt, rd, 0, st_nxt);
+                    if (s > kBar && (s - kBar - 1) % 4 == 1 && (s - kBar - 1) / 4 < kEarly)
+                        issue_load(t + 2, stage_cur, (s - kBar - 1) / 4);
                 }
                 KR_SCHED_FENCE();
             }
