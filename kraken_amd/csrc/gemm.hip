@@ -599,7 +599,7 @@ static int gemm_reduce(const void* A, int64_t lda_m, int64_t lda_k, const void* 
     g.peers_on_mfma = 1;
     if (const char* t = getenv("KRAKEN_AMD_GEMM_PEERS")) g.peers_on_mfma = t[0] == 'e' ? 0 : t[0] == 'f' ? 2 : t[0] == 'l' ? 3 : 1;
     // MFMA block shape of the 256x256 kernel's k loop: 16x16x32 draws less power per flop than
-    // 32x32x16 and the chip is power-limited (4-7 % faster with warm operands, same bits).  It
+    // 32x32x16 and the chip is power-limited (5-10 % faster with warm operands; results agree to fp32 rounding).  It
     // has no form that adds the peers on the matrix cores: its tiles add them in the epilogue,
     // which costs little while the band is a small part of the rows (8192x8192x3584 with a band
     // of 1024 rows: 367 -> 354 us) and much when every tile has peers (4096x8192x1024: 120 ->

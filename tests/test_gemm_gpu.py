@@ -242,6 +242,44 @@ def test_split_k_loop_replays_from_a_graph(dev):
             assert torch.equal(e, r)
 
 
+@pytest.mark.parametrize("b_t", [False, True])
+def test_both_mfma_block_shapes_agree(dev, monkeypatch, b_t):
+    """The 256 x 256 kernel's k loop on 16x16x32 blocks (default) and on 32x32x16 blocks: the same
+    products, summed 32 or 16 at a time inside the matrix cores, so the fp32 results agree to
+    rounding and the bf16 ones to an ulp -- for full and ragged shapes, the reduce-scatter form
+    and the split launches."""
+    monkeypatch.setenv("KRAKEN_AMD_GEMM_TILE", "256")
+    outs = {}
+    for mfma in ("16", "32"):
+        monkeypatch.setenv("KRAKEN_AMD_GEMM_MFMA", mfma)
+        res = []
+        for (M, N, K) in [(512, 768, 448), (520, 264, 192), (256, 256, 64)]:
+            a, b, _ = mk(M, N, K, 0, b_t, seed=K)
+            ad, bd = a.to(dev), b.to(dev)
+            res.append(fused.gemm_one_shot_all_reduce_fused(ad, bd))
+            res.append(fused.gemm_one_shot_all_reduce_fused(ad, bd, out_dtype=BF16))
+        M, N, K, W = 1024, 512, 256, 4
+        a, b, _ = mk(M, N, K, 0, b_t, seed=1)
+        peers = torch.stack([orc.randn_bf16((M // W, N), 100 + j) for j in range(W - 1)]).to(dev)
+        c_scratch = torch.zeros(M, N, dtype=BF16, device=dev)
+        res.append(fused.gemm_reduce_scatter(a.to(dev), b.to(dev), peers=peers, rank=2, c_scratch=c_scratch))
+        res.append(c_scratch)
+        monkeypatch.setenv("KRAKEN_AMD_GEMM_TAILSPLIT", "4")      # 6 tiles, every one split four ways
+        a, b, _ = mk(512, 768, 1024, 0, b_t, seed=2)
+        res.append(fused.gemm_one_shot_all_reduce_fused(a.to(dev), b.to(dev)))
+        monkeypatch.delenv("KRAKEN_AMD_GEMM_TAILSPLIT")
+        outs[mfma] = res
+    for x, y in zip(outs["16"], outs["32"]):
+        if x.dtype == torch.float32:
+            torch.testing.assert_close(x, y, rtol=1e-5, atol=1e-4)
+        else:
+            # two bf16 ulps: in the reduce-scatter form the 32x32x16 kernel adds the band's peers on
+            # the matrix cores (one rounding), the 16x16x32 kernel in the epilogue (product rounded first)
+            torch.testing.assert_close(x, y, rtol=1.6e-2, atol=1e-2)
+    a, b, _ = mk(512, 768, 448, 0, b_t, seed=448)
+    torch.testing.assert_close(outs["16"][0].cpu(), a.float() @ b.float(), rtol=1e-3, atol=1e-3)
+
+
 def _band_tile_counts(M, N, W, bm):
     rows = M // W
     return [(((r + 1) * rows - 1) // bm - (r * rows) // bm + 1) * -(-N // bm) for r in range(W)]
