@@ -446,11 +446,11 @@ __device__ __forceinline__ void gemm_dtl_tile(const GemmArgs& g, unsigned char* 
     __builtin_amdgcn_s_waitcnt(vmcnt_imm(kEarly));
     __builtin_amdgcn_s_barrier();
     KR_SCHED_FENCE();
-    if constexpr (MI16) {
-#pragma unroll
-        for (int i = 0; i < 2 * TM; ++i) read_a16(0, i, 0, 0);
+    if constexpr (MI16) {   // (A blocks 4..7 are read inside the first sub-step)
 #pragma unroll
         for (int j = 0; j < 2 * TN; ++j) read_b16(0, j, 0, 0);
+#pragma unroll
+        for (int i = 0; i < TM; ++i) read_a16(0, i, 0, 0);
     } else {
 #pragma unroll
         for (int i = 0; i < TM; ++i) read_a(0, i, 0, 0);
@@ -502,17 +502,27 @@ __device__ __forceinline__ void gemm_dtl_tile(const GemmArgs& g, unsigned char* 
     };
     // The same k-step on 16x16x32 blocks: two sub-steps of 64 MFMAs (32 k each) on alternating
     // fragment buffers.  An MFMA lasts 16 cycles here, room for about three other instructions,
-    // so fragment reads and loads are spread one per slot: during sub-step 0 the 16 fragments of
-    // sub-step 1 (every fourth MFMA; B blocks first, then the A blocks in the order the rows of
-    // MFMAs need them).  Behind MFMA 7 of sub-step 1 all of them have long returned: wait for the
-    // loads of step t+1, barrier; then, in slots of their own, the first fragments of step t+1 and
-    // 14 of the 16 loads of step t+2 into the stage just vacated (the last two follow at the start
-    // of the next step).
+    // so fragment reads and loads get MFMA slots of their own.  Row i of MFMAs needs A block i and
+    // all B blocks, so a sub-step can start on the B blocks and the first A blocks; the others
+    // follow while it runs.
+    //   sub-step 0: the fragments of sub-step 1 (every fourth slot), A blocks 4..7 of this
+    //     sub-step (slots 1, 9, 17, 25), the last two loads of step t+1 (slots 2, 6);
+    //   sub-step 1, behind MFMA 7: every LDS read of the stage has returned -- barrier (a): the
+    //     stage is free, the loads of step t+2 start (one per four MFMAs);
+    //   behind MFMA 47: wait for the loads of step t+1 (the ten younger ones of step t+2 stay
+    //     outstanding) -- barrier (b) -- and read the B blocks and A blocks 0..3 of step t+1.
+    // Two barriers instead of one buy the loads a third more time to arrive (from slot 9 of one
+    // step to slot 47 of the next): the wait sits right in front of the first read that needs
+    // the data, not in front of the first load that needs the room.
     constexpr int NM16 = 4 * TM * TN;
     auto read_frag16 = [&](int buf, int r, int ks2, uint32_t stage_off) __attribute__((always_inline)) {
         if (r < 2 * TN) read_b16(buf, r, ks2, stage_off);
         else read_a16(buf, r - 2 * TN, ks2, stage_off);
     };
+    constexpr int kBarA = 2 * TN - 1;      // last MFMA of the first row
+    constexpr int kBarB = 47;
+    constexpr int kLoadsBeforeB = (kBarB - kBarA - 2) / 4 + 1;   // loads of step t+2 in slots 9, 13, ... < kBarB
+    static_assert(!MI16 || (kLoadsBeforeB == 10 && kLoadsBeforeB <= kEarly), "wait count of barrier (b)");
     auto k_step16 = [&](int t, auto stage_c) __attribute__((always_inline)) {
         const uint32_t stage_cur = stage_c;
         const uint32_t stage_nxt = stage_cur ^ 1u;
@@ -531,22 +541,26 @@ __device__ __forceinline__ void gemm_dtl_tile(const GemmArgs& g, unsigned char* 
                              : "v"(bfr16[cur][j]), "v"(af16[cur][i]));
                 if (ks2 == 0) {
                     if (s % 4 == 0) read_frag16(nxt, s / 4, 1, st_cur);
+                    if (s % 8 == 1 && s / 8 + 4 < 2 * TM) read_a16(cur, s / 8 + 4, 0, st_cur);
                     // the last loads of step t+1
-                    if (s % 4 == 1 && s / 4 < LOADS_PER_TILE - kEarly) issue_load(t + 1, stage_nxt, kEarly + s / 4);
+                    if ((s == 2 || s == 6) && kEarly + s / 4 < LOADS_PER_TILE) issue_load(t + 1, stage_nxt, kEarly + s / 4);
                 } else {
-                    constexpr int kBar = 2 * TN - 1;   // last MFMA of the first row
-                    if (s == kBar) {
+                    if (s == kBarA) {
                         KR_SCHED_FENCE();
                         __builtin_amdgcn_s_waitcnt(kLgkm0);
-                        __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));
                         __builtin_amdgcn_s_barrier();
                     }
-                    // (slots 8, 11, 12, then every fourth from 15: none shared with a load)
-                    const int rd = s == kBar + 1 ? 0 : s == kBar + 4 ? 1 : s == kBar + 5 ? 2
-                                   : (s >= kBar + 8 && (s - kBar - 8) % 4 == 0) ? 3 + (s - kBar - 8) / 4 : -1;
-                    if (rd >= 0 && rd < 2 * (TM + TN)) read_frag16(nxt, rd, 0, st_nxt);
-                    if (s > kBar && (s - kBar - 1) % 4 == 1 && (s - kBar - 1) / 4 < kEarly)
-                        issue_load(t + 2, stage_cur, (s - kBar - 1) / 4);
+                    if (s > kBarA && (s - kBarA - 1) % 4 == 1 && (s - kBarA - 1) / 4 < kEarly)
+                        issue_load(t + 2, stage_cur, (s - kBarA - 1) / 4);
+                    if (s == kBarB) {
+                        KR_SCHED_FENCE();
+                        __builtin_amdgcn_s_waitcnt(vmcnt_imm(kLoadsBeforeB));
+                        __builtin_amdgcn_s_barrier();
+                    }
+                    // B blocks and A blocks 0..3 of k-step t+1: slots 48, 50, ..., 62; 63; 51, 55, 59
+                    if (s > kBarB && s % 2 == 0) read_frag16(nxt, (s - kBarB - 1) / 2, 0, st_nxt);
+                    if (s == NM16 - 1) read_frag16(nxt, 2 * TN, 0, st_nxt);
+                    if (s > kBarB && s % 4 == 3 && s < NM16 - 1) read_frag16(nxt, 2 * TN + 1 + (s - kBarB - 4) / 4, 0, st_nxt);
                 }
                 KR_SCHED_FENCE();
             }
