@@ -143,10 +143,11 @@ int kr_rmsnorm_bf16(const void* x, const void* w, float eps, int64_t rows, int64
  * bf16 result, tiles whose peers are added in the epilogue round the product
  * to bf16 before the sum, as gemm_reduce_scatter_fused.py:72 does.
  * Non-finite input: for shapes the 256x256 kernel takes (more than 128 tiles
- * of 256x256, K % 64 == 0) the peers of tiles lying wholly in the band are added
- * on the matrix cores, where an Inf/NaN in a peer also turns the rest of
- * the aligned 32-column block of its row into NaN; KRAKEN_AMD_GEMM_PEERS=epilogue
- * in the environment keeps such values in their own element.
+ * of 256x256, K % 64 == 0) and a band of at least half the rows, the peers of
+ * tiles lying wholly in the band are added on the matrix cores, where an
+ * Inf/NaN in a peer also turns the rest of the aligned 32-column block of its
+ * row into NaN; KRAKEN_AMD_GEMM_PEERS=epilogue in the environment keeps such
+ * values in their own element (as calls with a smaller band always do).
  *
  * Replaces
  *   kraken/fused/gemm_one_shot_all_reduce_fused.py:56-99   (band = all rows)
