@@ -489,6 +489,7 @@ def main() -> None:
                     help="--sweep: shapes, comma separated (e.g. 1024,6656,8192; a single number for all_reduce)")
     ap.add_argument("--world-size", type=int, default=8, help="--sweep: number of ranks whose buffers are reduced")
     ap.add_argument("--save-path", default=None, help="--sweep: also write the table as CSV")
+    ap.add_argument("--plot-path", default=None, help="--sweep: also plot time against shape, one line per backend (PNG)")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         _die_multi_gpu(max(args.gpus, int(os.environ.get("WORLD_SIZE", "1"))))
@@ -513,7 +514,7 @@ def main() -> None:
             shapes = [tuple(int(x) for x in sh.split(",")) for sh in args.shape]
             if args.sweep == "all_reduce":
                 shapes = [sh[0] for sh in shapes]
-        run_sweep(args.sweep, args.backend, shapes, args.world_size, args.save_path, dev=dev)
+        run_sweep(args.sweep, args.backend, shapes, args.world_size, args.save_path, dev=dev, plot_path=args.plot_path)
         return
 
     if args.calibrate_copy:

@@ -136,8 +136,10 @@ SWEEPS = {
 
 
 def run_sweep(name: str, backends: list[str] | None = None, shapes=None, world_size: int = 8,
-              save_path: str | None = None, iters: int = 25, dev=None) -> list[dict]:
-    """Run sweep ``name``; print the table; return one dict per shape."""
+              save_path: str | None = None, iters: int = 25, dev=None, plot_path: str | None = None) -> list[dict]:
+    """Run sweep ``name``; print the table; return one dict per shape.  ``plot_path``: also
+    draw the times against the shapes, one line per backend, as the reference's bias sweeps do
+    (``benchmark/benchmark_all_reduce_bias.py:150-154``)."""
     from tabulate import tabulate
 
     build, default_shapes, tol = SWEEPS[name]
@@ -168,6 +170,12 @@ def run_sweep(name: str, backends: list[str] | None = None, shapes=None, world_s
         for k, v in row.items():
             table[k].append(v)
     print(tabulate(table, headers="keys", tablefmt="github", floatfmt=".3f"))
+    if plot_path is not None:
+        from .utils import plot_experiment_comparison
+
+        names = backends or [k for k in rows[0] if k not in ("shape", "dtype", "world_size", "Best Backend")
+                             and not k.startswith("Speedup")]
+        plot_experiment_comparison([r["shape"] for r in rows], names, [[r[b] for b in names] for r in rows], plot_path)
     if save_path is not None:
         with open(save_path, "w", newline="") as f:
             wr = csv.DictWriter(f, fieldnames=list(rows[0].keys()))

@@ -282,6 +282,19 @@ def test_public_names_match_reference_layout():
         "two_shot_all_reduce_bias_rms_norm",
     }
     assert kraken_amd.__all__ == ["_lib", "_logging", "comm", "fused"]
+    # kraken/_logging/__init__.py:1-4 (the PTX dump helper has no counterpart: nothing is compiled at run time)
+    from kraken_amd import _logging
+    assert set(_logging.__all__) == {"benchmark_with_event", "benchmark_with_profiler", "plot_experiment_comparison"}
+
+
+def test_plot_experiment_comparison_writes_the_chart(tmp_path):
+    from kraken_amd._logging import plot_experiment_comparison
+    out = tmp_path / "sweep.png"
+    plot_experiment_comparison(["(1, 5k)", "(2, 5k)", "(4, 5k)"], ["hip", "torch"], [[6.3, 14.6], [6.3, 13.4], [6.4, 13.6]],
+                               str(out))
+    assert out.stat().st_size > 1000 and out.read_bytes()[:4] == b"\x89PNG"
+    with pytest.raises(AssertionError):
+        plot_experiment_comparison(["a"], ["x", "y"], [[1.0]], str(out))      # a row per size, a value per experiment
 
 
 def test_wrappers_assert_like_the_reference_and_refuse_host_tensors():

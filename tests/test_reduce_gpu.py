@@ -271,3 +271,19 @@ def test_reduce_paths_replay_from_a_graph(dev):
         torch.cuda.synchronize()
         for e, r in zip(eager, got):
             assert torch.equal(e, r)
+
+
+def test_benchmark_helpers(dev):
+    """The reference's two timing methods (kraken/_logging/benchmarking.py): per-call events and
+    profiler events matched by kernel name; both with the reference's keywords."""
+    from kraken_amd._logging import benchmark_with_event, benchmark_with_profiler
+    stack = orc.make_stack(8, (256, 4096)).to(dev)
+    fn = lambda: comm.one_shot_all_reduce(stack)                      # noqa: E731
+    t_event = benchmark_with_event(fn, warmup_iters=5, benchmark_iters=10, flush_l2=True)
+    t_graph = benchmark_with_event(fn, warmup_iters=5, benchmark_iters=10, flush_l2=False, cuda_graph=True)
+    t_index = benchmark_with_event(lambda i: comm.one_shot_all_reduce(stack), warmup_iters=2, benchmark_iters=5)
+    assert 0.5 < t_event < 500 and 0.5 < t_graph < 500 and 0.5 < t_index < 500
+    t_prof = benchmark_with_profiler(fn, r".*reduce_kernel.*", warmup_iters=5, benchmark_iters=10)
+    assert 0.5 < t_prof < 500
+    assert benchmark_with_profiler(fn, r"no such kernel", warmup_iters=1, benchmark_iters=2) == 0.0
+
