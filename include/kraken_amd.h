@@ -326,6 +326,21 @@ int kr_stream_wait_value32(const uint32_t* addr, uint32_t value, int64_t wait_li
                            int32_t* status, void* stream);
 
 /*
+ * The two flag primitives of the kernels above in one launch, for testing them on their own:
+ * `producers` workgroups each set flags[block] to 1 (release exchange), `consumers` further
+ * workgroups each wait until the flag of producer (block - producers) / (consumers / producers)
+ * reads 1 (acquire loads in a loop).  flags: uint32[producers] in device memory, zeroed by the
+ * caller.  A consumer whose flag does not come within wait_limit_us microseconds (0: 5 s)
+ * stores 1 + flag index to *status (device int32, may be NULL) and ends, so the launch always
+ * drains.  consumers % producers == 0.
+ * Replaces arrive_gmem_barrier / wait_gmem_barrier
+ * (kraken/_ptx_utils/gmem_barrier_arrive_wait.py:7-23, 26-68) as exercised by
+ * test/test_ptx_utils.py:80-116.
+ */
+int kr_flag_arrive_wait(uint32_t* flags, int producers, int consumers, int64_t wait_limit_us,
+                        int32_t* status, void* stream);
+
+/*
  * Stream-ordered device-to-device copy of `bytes` bytes that runs on the GPU's copy engines
  * (SDMA) and not as a copy kernel, so it takes no compute units from a GEMM running beside it.
  * Source and destination must not overlap.  bytes == 0: nothing is done.

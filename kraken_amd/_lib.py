@@ -87,6 +87,7 @@ _SIGNATURES = {
     ),
     "kr_stream_wait_value32": (c_int, [c_void_p, ctypes.c_uint32, c_int64, c_void_p, c_void_p]),
     "kr_copy_engine_memcpy": (c_int, [c_void_p, c_void_p, c_int64, c_void_p]),
+    "kr_flag_arrive_wait": (c_int, [c_void_p, c_int, c_int, c_int64, c_void_p, c_void_p]),
     "kr_reduce_rotated_bf16": (c_int, [c_void_p, c_int, c_int64, c_int64, c_int, c_int, c_void_p, c_void_p]),
 }
 

@@ -30,7 +30,45 @@ __global__ __launch_bounds__(kWave) void wait_value32_kernel(const uint32_t* add
     __atomic_thread_fence(__ATOMIC_ACQUIRE);
 }
 
+// The two flag primitives the kernels of the all-gather matmul and of the producer GEMM use, in
+// one launch: blocks 0 .. P-1 each set their flag (release exchange, as arrive_gmem_barrier with
+// op = atomic_xchg), every other block waits for the flag of producer (block - P) / (C / P)
+// (acquire load in a loop, as wait_gmem_barrier) -- bounded by `ticks`, after which the block
+// stores 1 + flag index to *status and ends.
+__global__ __launch_bounds__(kWave) void flag_arrive_wait_kernel(uint32_t* flags, int producers, int consumers,
+                                                                uint64_t ticks, int* status) {
+    const int b = blockIdx.x;
+    if (b < producers) {
+        if (threadIdx.x == 0) __hip_atomic_exchange(flags + b, 1u, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
+        return;
+    }
+    const int p = (b - producers) / (consumers / producers);
+    const uint64_t t0 = __builtin_amdgcn_s_memrealtime();
+    while (__hip_atomic_load(flags + p, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_AGENT) != 1u) {
+        if (__builtin_amdgcn_s_memrealtime() - t0 > ticks) {
+            if (status != nullptr && threadIdx.x == 0)
+                __hip_atomic_store(status, 1 + p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            break;
+        }
+        __builtin_amdgcn_s_sleep(16);
+    }
+}
+
 }  // namespace kr
+
+extern "C" int kr_flag_arrive_wait(uint32_t* flags, int producers, int consumers, int64_t wait_limit_us, int* status,
+                                   void* stream) {
+    if (producers < 1 || consumers < 0 || producers > 4096 || consumers > 65536) return KR_ERR_BAD_DIM;
+    if (consumers % producers != 0) return KR_ERR_STRIPE;
+    if (flags == nullptr) return KR_ERR_NULL_POINTER;
+    if ((reinterpret_cast<uintptr_t>(flags) & 3u) != 0 || (reinterpret_cast<uintptr_t>(status) & 3u) != 0)
+        return KR_ERR_ALIGNMENT;
+    if (wait_limit_us < 0) return KR_ERR_BAD_DIM;
+    const uint64_t ticks = (uint64_t)(wait_limit_us > 0 ? wait_limit_us : 5000000) * 100u;
+    hipLaunchKernelGGL(kr::flag_arrive_wait_kernel, dim3((unsigned)(producers + consumers)), dim3(kr::kWave), 0,
+                       (hipStream_t)stream, flags, producers, consumers, ticks, status);
+    return (int)hipGetLastError();
+}
 
 extern "C" int kr_stream_write_value32(uint32_t* addr, uint32_t value, void* stream) {
     if (addr == nullptr) return KR_ERR_NULL_POINTER;

@@ -221,6 +221,11 @@ def test_gemm_producer_argument_errors(lib):
     assert g(FAKE + 2, 1, 0, None, None) == _lib.KR_ERR_ALIGNMENT
     assert g(FAKE, 1, 0, FAKE + 1, None) == _lib.KR_ERR_ALIGNMENT
     assert g(FAKE, 1, -5, None, None) == _lib.KR_ERR_BAD_DIM
+    k = lib.kr_flag_arrive_wait
+    assert k(None, 8, 32, 0, None, None) == _lib.KR_ERR_NULL_POINTER
+    assert k(FAKE, 0, 32, 0, None, None) == _lib.KR_ERR_BAD_DIM
+    assert k(FAKE, 8, 30, 0, None, None) == _lib.KR_ERR_STRIPE          # consumers per producer must be whole
+    assert k(FAKE + 2, 8, 32, 0, None, None) == _lib.KR_ERR_ALIGNMENT
     h = lib.kr_copy_engine_memcpy
     assert h(FAKE, FAKE + 64, -1, None) == _lib.KR_ERR_BAD_DIM
     assert h(None, None, 0, None) == 0                        # nothing to copy

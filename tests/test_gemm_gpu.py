@@ -360,6 +360,25 @@ def test_copies_on_the_copy_engines(dev):
     assert status.item() == 0 and torch.equal(sent.view(W * m, N), gemm_out)
 
 
+def test_flag_arrive_wait(dev):
+    """test/test_ptx_utils.py:80-116: 8 producer workgroups set their flags, 32 consumers wait for
+    them in the same launch; the flags end as 1 and no consumer runs into the limit."""
+    lib = _lib.load()
+    stream = torch.cuda.current_stream(dev).cuda_stream
+    flags = torch.zeros(64, dtype=torch.int32, device=dev)
+    status = torch.zeros(1, dtype=torch.int32, device=dev)
+    _lib.check(lib.kr_flag_arrive_wait(flags.data_ptr(), 8, 32, 0, status.data_ptr(), stream), "flag_arrive_wait")
+    torch.cuda.synchronize()
+    expect = torch.zeros_like(flags)
+    expect[:8] = 1
+    assert torch.equal(flags, expect) and status.item() == 0
+    # one producer, four consumers, on a flag further into the array
+    flags.zero_()
+    _lib.check(lib.kr_flag_arrive_wait(flags.data_ptr() + 4, 1, 4, 2000, status.data_ptr(), stream), "flag_arrive_wait")
+    torch.cuda.synchronize()
+    assert flags.tolist() == [0, 1] + [0] * 62 and status.item() == 0
+
+
 def test_copy_engine_scatter_wait_is_bounded(dev):
     """A flag that never comes: the stream-ordered wait gives up after its limit, records it in
     `status`, and the stream drains."""
