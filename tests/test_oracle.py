@@ -245,3 +245,26 @@ def test_all_gather_matmul_exact_gather():
     a_full, c = orc.all_gather_matmul(stack, b)
     assert torch.equal(a_full, torch.cat(list(stack), 0))
     torch.testing.assert_close(c.float(), torch.cat([s.float() @ b.float() for s in stack], 0), rtol=2 ** -7, atol=1e-5)
+
+
+def test_known_answers_of_the_reference_tests():
+    """tests/golden/known_answers.json: the closed-form cases of the reference's tests, against the oracle."""
+    import json
+    import pathlib
+
+    cases = {c["name"]: c for c in json.loads((pathlib.Path(__file__).parent / "golden" / "known_answers.json").read_text())["cases"]}
+    c = cases["gemm_all_reduce_rank_specific"]
+    W, M, N, K = c["world_size"], c["M"], c["N"], c["K"]
+    b = torch.ones(K, N, dtype=torch.bfloat16)
+    partials = [(torch.full((M, K), float(r + 1), dtype=torch.bfloat16).float() @ b.float()).to(torch.bfloat16) for r in range(W)]
+    out = orc.gemm_all_reduce(torch.full((M, K), 1.0, dtype=torch.bfloat16), b, torch.stack(partials[1:]))
+    torch.testing.assert_close(out, torch.full((M, N), c["expected_value"]), rtol=c["tolerance"], atol=c["tolerance"])
+    c = cases["gemm_reduce_scatter_rank_specific"]
+    W, M, N, K = c["world_size"], c["M"], c["N"], c["K"]
+    b = torch.ones(K, N, dtype=torch.bfloat16)
+    for rank in range(W):
+        a = torch.full((M, K), float(rank + 1), dtype=torch.bfloat16)
+        peers = torch.stack([torch.full((M // W, N), float((r + 1) * K), dtype=torch.bfloat16) for r in range(W) if r != rank])
+        out, _ = orc.gemm_reduce_scatter(a, b, peers, rank, W)
+        assert torch.equal(out.float(), torch.full((M // W, N), c["expected_value"]))
+
