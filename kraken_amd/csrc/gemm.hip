@@ -464,11 +464,14 @@ static int64_t gemm_dtl_tail_workspace_bytes(int tail_tiles, int splits) {
 // (M = 512, K = 16384: 200 -> 146 us; M = 1024, K = 32768: 622 -> 434 us) except 104 tiles at
 // K = 4096; transposed-contiguous B only with much work per tile (52 tiles at K = 32768
 // 308 -> 279 us, 104 tiles at K = 16384 287 -> 281 us; below that up to 15 % slower).
-static bool whole_launch_split_pays(int64_t M, int64_t N, int64_t K, bool b_nt) {
+// (plain: a product without peers, band or second output.  There the finishing pass only sums and
+// stores, and with the 16x16x32 kernels transposed B pays from 48 tiles and K = 8192 on: 52 tiles
+// 99 -> 94 us, 104 tiles 144 -> 139 us; with a reduce-scatter epilogue the same shapes lose 5-10 %.)
+static bool whole_launch_split_pays(int64_t M, int64_t N, int64_t K, bool b_nt, bool plain) {
     if (M <= 0 || N <= 0 || M % 256 != 0 || N % 256 != 0 || K % 64 != 0) return false;
     const int64_t tiles = (M / 256) * (N / 256);
     if (tiles < 24 || tiles > 128) return false;
-    if (b_nt) return tiles * K >= (int64_t)52 * 32768;
+    if (b_nt) return tiles * K >= (int64_t)52 * 32768 || (plain && tiles >= 48 && K >= 8192);
     return K >= 8192 || (K >= 4096 && tiles <= 64);
 }
 
@@ -575,7 +578,7 @@ static int gemm_reduce(const void* A, int64_t lda_m, int64_t lda_k, const void* 
     // faster from 144 tiles on and 5-10 % slower at 128, for K from 1024 to 8192.
     bool big = ((M + 255) / 256) * ((N + 255) / 256) > 128 && K >= 256;
     // (few rows and a long K loop: the large tile again, with every tile's K loop split)
-    if (!big && workspace != nullptr && gather == nullptr && whole_launch_split_pays(M, N, K, b_nt)) {
+    if (!big && workspace != nullptr && gather == nullptr && whole_launch_split_pays(M, N, K, b_nt, n_peers == 0 && c_full == nullptr && bias == nullptr)) {
         int tail, ts;
         tail_split_plan((M / 256) * (N / 256), K, &tail, &ts);
         big = tail > 0 && gemm_dtl_tail_workspace_bytes(tail, ts) <= workspace_bytes;
@@ -758,7 +761,7 @@ extern "C" int64_t kr_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K) {
     const int S = split_k_factor(tiles, K);
     int64_t bytes = S > 1 ? split_k_workspace_bytes(M, N, S) : 0;
     // the layout of B is not known here: enough for either kernel
-    if (force_tile == nullptr && (whole_launch_split_pays(M, N, K, true) || whole_launch_split_pays(M, N, K, false))) {
+    if (force_tile == nullptr && (whole_launch_split_pays(M, N, K, true, true) || whole_launch_split_pays(M, N, K, false, true))) {
         int tail, ts;
         tail_split_plan((M / 256) * (N / 256), K, &tail, &ts);
         if (tail > 0) bytes = std::max(bytes, gemm_dtl_tail_workspace_bytes(tail, ts));
