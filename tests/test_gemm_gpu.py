@@ -280,6 +280,21 @@ def test_both_mfma_block_shapes_agree(dev, monkeypatch, b_t):
     torch.testing.assert_close(outs["16"][0].cpu(), a.float() @ b.float(), rtol=1e-3, atol=1e-3)
 
 
+@pytest.mark.parametrize("b_t", [False, True])
+@pytest.mark.parametrize("mfma", ["16", "32"])
+def test_split_parts_of_very_few_k_steps(dev, monkeypatch, b_t, mfma):
+    """Forced splits that leave a workgroup one or two k-steps (and uneven shares): the prologue,
+    the loads past the end and the waits of the k loop must still line up."""
+    monkeypatch.setenv("KRAKEN_AMD_GEMM_TILE", "256")
+    monkeypatch.setenv("KRAKEN_AMD_GEMM_MFMA", mfma)
+    for (M, N, K, S) in [(512, 768, 256, 4), (512, 768, 192, 3), (256, 256, 64, 1), (512, 512, 128, 2), (768, 512, 320, 5),
+                         (512, 768, 448, 2)]:
+        monkeypatch.setenv("KRAKEN_AMD_GEMM_TAILSPLIT", str(S))
+        a, b, _ = mk(M, N, K, 0, b_t, seed=S)
+        out = fused.gemm_one_shot_all_reduce_fused(a.to(dev), b.to(dev))
+        torch.testing.assert_close(out.cpu(), a.float() @ b.float(), rtol=1e-3, atol=1e-3)
+
+
 def _band_tile_counts(M, N, W, bm):
     rows = M // W
     return [(((r + 1) * rows - 1) // bm - (r * rows) // bm + 1) * -(-N // bm) for r in range(W)]
