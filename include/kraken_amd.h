@@ -44,6 +44,7 @@ extern "C" {
 #define KR_ERR_BAND          -8  /* row band outside [0, M) or M % W != 0           */
 #define KR_ERR_LAYOUT        -9  /* operand strides not supported                   */
 #define KR_ERR_STRIPE       -10  /* stripe block not a multiple of 8 / bad rank     */
+#define KR_ERR_SCRATCH      -11  /* shape needs more than KR_STATIC_SCRATCH_BYTES   */
 
 #define KR_MAX_WORLD 16
 #define KR_MAX_ROW   65536
@@ -245,6 +246,31 @@ int kr_gemm_reduce_ptrs_ws_bf16(const void* A, int64_t lda_m, int64_t lda_k,
                                 void* c_full, void* out, int out_is_fp32,
                                 int64_t tile_pivot,
                                 void* workspace, int64_t workspace_bytes, void* stream);
+
+/*
+ * kr_gemm_reduce_ws_bf16 for callers that can neither allocate a workspace nor let the library
+ * allocate: code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.
+ * It has no counterpart in the reference.  Arguments, arithmetic, tile choice and results are
+ * those of kr_gemm_reduce_ws_bf16 called with a workspace of KR_STATIC_SCRATCH_BYTES bytes
+ * (bit-identical output); the workspace is a device array inside the library (64 MiB of device
+ * memory on every GPU the library is used on, held until the process ends), looked up once per
+ * device, and the call performs no allocation of any kind.  A shape whose split would need more
+ * (kr_gemm_workspace_bytes(M, N, K) > KR_STATIC_SCRATCH_BYTES) is refused with KR_ERR_SCRATCH
+ * before anything is launched; shapes that are not split use no scratch at all.  Every call on
+ * one GPU shares that GPU's array: calls that may overlap (different streams without an
+ * ordering between them, or several host threads) race on it and must be serialised by the
+ * caller.  Nothing in the array has to start at zero (the first launch overwrites every word
+ * the second reads), so a call leaves nothing behind that a later call depends on.
+ */
+#define KR_STATIC_SCRATCH_BYTES (64ll << 20)
+int kr_gemm_reduce_noalloc_bf16(const void* A, int64_t lda_m, int64_t lda_k,
+                                const void* B, int64_t ldb_k, int64_t ldb_n,
+                                int64_t M, int64_t N, int64_t K,
+                                const void* peers, int n_peers, int64_t peers_stride,
+                                const void* bias,
+                                int64_t band_row0, int64_t band_rows,
+                                void* c_full, void* out, int out_is_fp32,
+                                int64_t tile_pivot, void* stream);
 
 /*
  * All-gather matmul that consumes A while it is still arriving:  C[M,N] = A[M,K] @ B[K,N]  (bf16, fp32

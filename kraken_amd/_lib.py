@@ -21,6 +21,7 @@ KR_ERR_ROW_TOO_LONG = -7
 KR_ERR_BAND = -8
 KR_ERR_LAYOUT = -9
 KR_ERR_STRIPE = -10
+KR_ERR_SCRATCH = -11
 
 _SIGNATURES = {
     "kr_version": (c_int, []),
@@ -57,6 +58,11 @@ _SIGNATURES = {
     ),
     "kr_rmsnorm_bf16": (c_int, [c_void_p, c_void_p, c_float, c_int64, c_int64, c_void_p, c_void_p]),
     "kr_gemm_reduce_bf16": (
+        c_int,
+        [c_void_p, c_int64, c_int64, c_void_p, c_int64, c_int64, c_int64, c_int64, c_int64,
+         c_void_p, c_int, c_int64, c_void_p, c_int64, c_int64, c_void_p, c_void_p, c_int, c_int64, c_void_p],
+    ),
+    "kr_gemm_reduce_noalloc_bf16": (
         c_int,
         [c_void_p, c_int64, c_int64, c_void_p, c_int64, c_int64, c_int64, c_int64, c_int64,
          c_void_p, c_int, c_int64, c_void_p, c_int64, c_int64, c_void_p, c_void_p, c_int, c_int64, c_void_p],

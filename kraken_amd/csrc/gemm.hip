@@ -24,6 +24,7 @@
 #include <type_traits>
 
 #include <algorithm>
+#include <mutex>
 
 #include "gemm_common.h"
 
@@ -478,6 +479,30 @@ static bool whole_launch_split_pays(int64_t M, int64_t N, int64_t K, bool b_nt, 
 // workspace of the two-pass form: S fp32 partial products of the whole [M, N] result
 static int64_t split_k_workspace_bytes(int64_t M, int64_t N, int S) { return (int64_t)S * M * N * 4; }
 
+// ---- the workspace form for callers that cannot allocate ------------------------------------------
+// The split-K workspace lives in a device array of the library instead of caller memory.  Host code
+// never uses the array's name as an address: each device's copy is looked up once, with that device
+// current, and the pointer kept is what the kernels get, exactly as they get the caller's workspace.
+static __device__ __align__(256) unsigned char scratch[KR_STATIC_SCRATCH_BYTES];
+
+constexpr int kMaxDevices = 64;
+static int static_scratch(void** out) {
+    static std::mutex mu;
+    static void* ptr_of_device[kMaxDevices] = {};
+    int dev = -1;
+    if (hipError_t e = hipGetDevice(&dev); e != hipSuccess) return (int)e;
+    if (dev < 0 || dev >= kMaxDevices) return (int)hipErrorInvalidDevice;
+    std::lock_guard<std::mutex> lock(mu);
+    if (ptr_of_device[dev] == nullptr) {
+        void* ptr = nullptr;
+        if (hipError_t e = hipGetSymbolAddress((void**)&ptr, HIP_SYMBOL(scratch)); e != hipSuccess) return (int)e;
+        if (ptr == nullptr) return (int)hipErrorInvalidSymbol;
+        ptr_of_device[dev] = ptr;
+    }
+    *out = ptr_of_device[dev];
+    return KR_OK;
+}
+
 // What the kernel exchanges with other streams while it runs (null pointer to gemm_reduce:
 // nothing): the arrival flags of the all-gather matmul (progress == nullptr: A is complete) and
 // the per-band counters of the producer GEMM (band_counter == nullptr: none).
@@ -501,7 +526,7 @@ static int gemm_reduce(const void* A, int64_t lda_m, int64_t lda_k, const void* 
                        const void* const* peer_ptrs, int64_t peers_stride, const void* bias,
                        int64_t band_row0, int64_t band_rows, void* c_full, void* out, int out_is_fp32,
                        int64_t tile_pivot, void* stream, const GatherSpec* gather = nullptr,
-                       void* workspace = nullptr, int64_t workspace_bytes = 0) {
+                       void* workspace = nullptr, int64_t workspace_bytes = 0, bool static_ws = false) {
     if (M < 0 || N < 0 || K < 0 || M > 0x7fffffffLL || N > 0x7fffffffLL || K > 0x7fffffffLL)
         return KR_ERR_BAD_DIM;
     if (n_peers < 0 || n_peers >= KR_MAX_WORLD) return KR_ERR_WORLD_SIZE;
@@ -520,6 +545,12 @@ static int gemm_reduce(const void* A, int64_t lda_m, int64_t lda_k, const void* 
     if (lda_m % 8 != 0 || ldb % 8 != 0) return KR_ERR_ALIGNMENT;
     if (!aligned16(A) || !aligned16(B) || !aligned16(bias) || !aligned16(c_full) || !aligned16(out))
         return KR_ERR_ALIGNMENT;
+    // (arguments are checked; a shape that is split now gets the library's own workspace)
+    if (static_ws && kr_gemm_workspace_bytes(M, N, K) > 0) {
+        const int rc = static_scratch(&workspace);
+        if (rc != KR_OK) return rc;
+        workspace_bytes = KR_STATIC_SCRATCH_BYTES;
+    }
 
     GemmArgs g;
     if (peer_ptrs != nullptr) {
@@ -790,4 +821,16 @@ extern "C" int kr_gemm_reduce_ptrs_ws_bf16(const void* A, int64_t lda_m, int64_t
     return gemm_reduce(A, lda_m, lda_k, B, ldb_k, ldb_n, M, N, K, peers, n_peers,
                        peers != nullptr ? peers : kNoPeers, 0, bias, band_row0, band_rows, c_full, out,
                        out_is_fp32, tile_pivot, stream, nullptr, workspace, workspace_bytes);
+}
+
+extern "C" int kr_gemm_reduce_noalloc_bf16(const void* A, int64_t lda_m, int64_t lda_k, const void* B,
+                                           int64_t ldb_k, int64_t ldb_n, int64_t M, int64_t N, int64_t K,
+                                           const void* peers, int n_peers, int64_t peers_stride,
+                                           const void* bias, int64_t band_row0, int64_t band_rows,
+                                           void* c_full, void* out, int out_is_fp32, int64_t tile_pivot,
+                                           void* stream) {
+    if (kr_gemm_workspace_bytes(M, N, K) > KR_STATIC_SCRATCH_BYTES) return KR_ERR_SCRATCH;
+    return gemm_reduce(A, lda_m, lda_k, B, ldb_k, ldb_n, M, N, K, peers, n_peers, nullptr, peers_stride, bias,
+                       band_row0, band_rows, c_full, out, out_is_fp32, tile_pivot, stream, nullptr, nullptr, 0,
+                       /*static_ws=*/true);
 }

@@ -16,6 +16,7 @@ extern "C" const char* kr_strerror(int code) {
         case KR_ERR_BAND: return "row band outside [0, M)";
         case KR_ERR_LAYOUT: return "operand strides not supported (A must be k-contiguous; B row-major or transposed-contiguous)";
         case KR_ERR_STRIPE: return "stripe block must be a positive multiple of 8 and 0 <= rank < W";
+        case KR_ERR_SCRATCH: return "the shape's split needs more scratch than the library's static device buffer (64 MiB) holds";
         default: break;
     }
     if (code > 0) return hipGetErrorString((hipError_t)code);

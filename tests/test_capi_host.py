@@ -247,6 +247,23 @@ def test_gemm_workspace_entries(lib):
              FAKE, need, None) == _lib.KR_ERR_NULL_POINTER
 
 
+def test_gemm_noalloc_entry_checks_arguments_first(lib, monkeypatch):
+    """The allocation-free form validates like the others (nothing is looked up or launched for
+    a rejected call) and refuses a split that its static scratch cannot hold."""
+    f = lib.kr_gemm_reduce_noalloc_bf16
+    base = (FAKE, 4096, 1, FAKE, 6656, 1, 128, 6656, 4096, None, 0, 0, None, 0, 128, None, FAKE, 0, 0)
+    assert f(FAKE, 4096, 2, *base[3:], None) == _lib.KR_ERR_LAYOUT
+    assert f(None, *base[1:], None) == _lib.KR_ERR_NULL_POINTER
+    assert f(FAKE + 4, *base[1:], None) == _lib.KR_ERR_ALIGNMENT
+    assert f(*base[:6], 0, 6656, 4096, None, 0, 0, None, 0, 0, None, FAKE, 0, 0, None) == 0   # M == 0: nothing to do
+    monkeypatch.setenv("KRAKEN_AMD_GEMM_TILE", "128")
+    monkeypatch.setenv("KRAKEN_AMD_GEMM_SPLITK", "16")                  # 16 partial products of 1024 x 2048 fp32
+    assert lib.kr_gemm_workspace_bytes(1024, 2048, 4096) == 16 * 1024 * 2048 * 4 > (64 << 20)
+    assert f(FAKE, 4096, 1, FAKE, 2048, 1, 1024, 2048, 4096, None, 0, 0, None, 0, 1024, None, FAKE, 0, 0,
+             None) == _lib.KR_ERR_SCRATCH
+    assert "scratch" in _lib.strerror(_lib.KR_ERR_SCRATCH)
+
+
 def test_striped_share_numel(lib):
     f = lib.kr_striped_share_numel
     numel, W, block = 8 * 37, 4, 16
