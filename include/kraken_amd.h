@@ -55,6 +55,10 @@ int kr_version(void);
 /* Human-readable text for a return code of this library (never NULL). */
 const char* kr_strerror(int code);
 
+/* The KRAKEN_AMD_* environment switches (testing and tuning) are read once per process, on the
+ * first call that consults them; this reads them again. */
+void kr_reload_env(void);
+
 /*
  * W-way elementwise reduce with optional bias.
  *   out[i] = bf16( [bias] + sum_{r=0..W-1} fp32(stack[r*slice_stride + i]) ),  0 <= i < numel
@@ -112,6 +116,31 @@ int64_t kr_striped_share_numel(int64_t numel, int W, int64_t stripe_block, int r
 int kr_reduce_rmsnorm_bf16(const void* stack, int W, int64_t slice_stride, int64_t rows, int64_t D,
                            const void* bias, int bias_is_vector, const void* w, float eps,
                            void* y, void* stream);
+
+/*
+ * kr_reduce_rmsnorm_bf16 / kr_reduce_rmsnorm_ptrs_bf16 with a workspace, for a few long rows
+ * (decode shapes: up to 64 rows whose W * D * 2 input bytes make one compute unit's intake the
+ * kernel's time).  A row is then spread over many compute units, one wavefront per 512 elements,
+ * and the wavefronts of a row exchange their partial sums of squares through the workspace and add
+ * them in a fixed order (results are reproducible run to run and equal the one-workgroup form up
+ * to the fp32 rounding of that order).
+ * `workspace`: device memory, 16-byte aligned, of at least kr_rmsnorm_workspace_bytes(W, rows, D)
+ * bytes (0: this shape is not split; the value does not depend on the shape otherwise, so one
+ * buffer serves every call).  It must be ZERO before its first use and is afterwards kept
+ * consistent by the kernels themselves (no clearing between calls, also not between replays of a
+ * captured graph; clearing it again between calls is harmless).  Calls that use one workspace
+ * must not overlap (same stream, or otherwise ordered).  workspace == NULL, a workspace that is
+ * too small, or a shape that does not profit: exactly the entry point without workspace.
+ * No counterpart in the reference (one 1024-thread CTA per row whatever the shape,
+ * kraken/fused/one_shot_all_reduce_bias_rms_norm.py:144-145).
+ */
+int64_t kr_rmsnorm_workspace_bytes(int W, int64_t rows, int64_t D);
+int kr_reduce_rmsnorm_ws_bf16(const void* stack, int W, int64_t slice_stride, int64_t rows, int64_t D,
+                              const void* bias, int bias_is_vector, const void* w, float eps,
+                              void* y, void* workspace, int64_t workspace_bytes, void* stream);
+int kr_reduce_rmsnorm_ptrs_ws_bf16(const void* const* bufs, int W, int64_t rows, int64_t D,
+                                   const void* bias, int bias_is_vector, const void* w, float eps,
+                                   void* y, void* workspace, int64_t workspace_bytes, void* stream);
 
 /*
  * Stand-alone RMSNorm: y = bf16( x * rsqrt(mean(x^2) + eps) * w ), row-wise.

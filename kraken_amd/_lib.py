@@ -26,6 +26,7 @@ KR_ERR_SCRATCH = -11
 _SIGNATURES = {
     "kr_version": (c_int, []),
     "kr_strerror": (c_char_p, [c_int]),
+    "kr_reload_env": (None, []),
     "kr_reduce_bf16": (
         c_int,
         [c_void_p, c_int, c_int64, c_int64, c_void_p, c_int64, c_int64, c_int, c_void_p, c_void_p],
@@ -55,6 +56,17 @@ _SIGNATURES = {
     "kr_reduce_rmsnorm_bf16": (
         c_int,
         [c_void_p, c_int, c_int64, c_int64, c_int64, c_void_p, c_int, c_void_p, c_float, c_void_p, c_void_p],
+    ),
+    "kr_rmsnorm_workspace_bytes": (c_int64, [c_int, c_int64, c_int64]),
+    "kr_reduce_rmsnorm_ws_bf16": (
+        c_int,
+        [c_void_p, c_int, c_int64, c_int64, c_int64, c_void_p, c_int, c_void_p, c_float, c_void_p,
+         c_void_p, c_int64, c_void_p],
+    ),
+    "kr_reduce_rmsnorm_ptrs_ws_bf16": (
+        c_int,
+        [c_void_p, c_int, c_int64, c_int64, c_void_p, c_int, c_void_p, c_float, c_void_p,
+         c_void_p, c_int64, c_void_p],
     ),
     "kr_rmsnorm_bf16": (c_int, [c_void_p, c_void_p, c_float, c_int64, c_int64, c_void_p, c_void_p]),
     "kr_gemm_reduce_bf16": (
@@ -122,6 +134,11 @@ def load() -> ctypes.CDLL:
             fn.argtypes = argtypes
         _lib = lib
     return _lib
+
+
+def reload_env() -> None:
+    """Make the library read the KRAKEN_AMD_* environment switches again (it reads them once)."""
+    load().kr_reload_env()
 
 
 def strerror(code: int) -> str:

@@ -78,11 +78,30 @@ class PeerBuffers:
 
     def reduce_rmsnorm(self, rows, D, bias_ptr, bias_is_vector, w_ptr, eps, y_ptr, stream) -> int:
         lib = _lib.load()
+        ws = row_workspace(self.tensors[0].device, lib.kr_rmsnorm_workspace_bytes(self.W, rows, D))
+        ws_ptr, ws_bytes = (ws.data_ptr(), ws.numel()) if ws is not None else (None, 0)
         if self.stacked is not None:
-            return lib.kr_reduce_rmsnorm_bf16(self.stacked.data_ptr(), self.W, self.stride, rows, D, bias_ptr,
-                                              bias_is_vector, w_ptr, eps, y_ptr, stream)
-        return lib.kr_reduce_rmsnorm_ptrs_bf16(self._table(0), self.W, rows, D, bias_ptr, bias_is_vector,
-                                               w_ptr, eps, y_ptr, stream)
+            return lib.kr_reduce_rmsnorm_ws_bf16(self.stacked.data_ptr(), self.W, self.stride, rows, D, bias_ptr,
+                                                 bias_is_vector, w_ptr, eps, y_ptr, ws_ptr, ws_bytes, stream)
+        return lib.kr_reduce_rmsnorm_ptrs_ws_bf16(self._table(0), self.W, rows, D, bias_ptr, bias_is_vector,
+                                                  w_ptr, eps, y_ptr, ws_ptr, ws_bytes, stream)
+
+
+_row_workspaces: dict[tuple[int, int], torch.Tensor] = {}
+
+
+def row_workspace(dev: torch.device, nbytes: int) -> torch.Tensor | None:
+    """Workspace of the split-row RMSNorm kernel: one zero-initialised buffer per (device, stream),
+    so that calls on different streams never share one; the kernels keep it consistent afterwards."""
+    if nbytes <= 0:
+        return None
+    key = (dev.index if dev.index is not None else torch.cuda.current_device(),
+           torch.cuda.current_stream(dev).cuda_stream)
+    ws = _row_workspaces.get(key)
+    if ws is None or ws.numel() < nbytes:
+        ws = torch.zeros(nbytes, dtype=torch.uint8, device=dev)
+        _row_workspaces[key] = ws
+    return ws
 
 
 def check_stack(stacked: torch.Tensor | Sequence[torch.Tensor]) -> PeerBuffers:

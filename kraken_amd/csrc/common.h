@@ -116,6 +116,22 @@ struct StackedPeers {
     __device__ __forceinline__ const u32x4* at(int r) const { return base + r * stride_v; }
 };
 
+// ---- tuning switches ----------------------------------------------------------
+// The KRAKEN_AMD_* environment variables (testing and tuning), read once per process and not on
+// every launch; kr_reload_env() reads them again.  -1 = not set.
+struct EnvSwitches {
+    int row_vpt;         // KRAKEN_AMD_ROW_VPT=1|2|4|8
+    int row_lat;         // KRAKEN_AMD_ROW_LAT=0|1
+    int row_split;       // KRAKEN_AMD_ROW_SPLIT=0|1
+    int gemm_tile;       // KRAKEN_AMD_GEMM_TILE=128|256 -> 128, 256
+    int gemm_peers;      // KRAKEN_AMD_GEMM_PEERS=epilogue|mfma|first|last -> 0, 1, 2, 3
+    int gemm_mfma;       // KRAKEN_AMD_GEMM_MFMA=16|32 -> 16, 32
+    int gemm_group;      // KRAKEN_AMD_GEMM_GROUP=<n>
+    int gemm_splitk;     // KRAKEN_AMD_GEMM_SPLITK=<n>
+    int gemm_tailsplit;  // KRAKEN_AMD_GEMM_TAILSPLIT=<n>
+};
+const EnvSwitches& env_switches();   // status.hip
+
 // ---- host-side checks -------------------------------------------------------
 static inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 

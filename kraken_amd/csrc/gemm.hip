@@ -418,10 +418,8 @@ using namespace kr;
 constexpr int kMaxSplits = 16;
 constexpr int kMinSplitSteps = 8;
 static int split_k_factor(int64_t tiles, int64_t K) {
-    if (const char* t = getenv("KRAKEN_AMD_GEMM_SPLITK")) {   // testing and tuning
-        const int v = atoi(t);
-        if (v >= 1 && v <= kMaxSplits) return (int)std::min<int64_t>(v, std::max<int64_t>(1, (K + BK - 1) / BK));
-    }
+    if (const int v = env_switches().gemm_splitk; v >= 1 && v <= kMaxSplits)   // testing and tuning
+        return (int)std::min<int64_t>(v, std::max<int64_t>(1, (K + BK - 1) / BK));
     // (up to 256 tiles a second workgroup per tile still finds a place next to the first; it pays
     // once the K loop is long: 208 tiles at K = 16384 measured 197 -> 178 us, at K = 4096 54 -> 62 us)
     if (tiles > 128 && tiles <= 256 && K >= 12288) return 2;
@@ -440,8 +438,7 @@ constexpr int kMaxTailSplits = 8;
 static void tail_split_plan(int64_t tiles, int64_t K, int* tail_out, int* splits_out) {
     *tail_out = 0;
     *splits_out = 1;
-    int64_t force = -1;
-    if (const char* t = getenv("KRAKEN_AMD_GEMM_TAILSPLIT")) force = atoi(t);   // 0: off, n: n parts (testing)
+    const int64_t force = env_switches().gemm_tailsplit;   // 0: off, n: n parts (testing)
     if (force == 0 || (tiles > 128 && tiles <= 256)) return;
     // up to 128 tiles the whole launch is one partial round
     const int64_t tail = tiles % 256;
@@ -615,10 +612,8 @@ static int gemm_reduce(const void* A, int64_t lda_m, int64_t lda_k, const void* 
         big = tail > 0 && gemm_dtl_tail_workspace_bytes(tail, ts) <= workspace_bytes;
     }
     // KRAKEN_AMD_GEMM_TILE=128|256 overrides the choice (testing and tuning)
-    if (const char* t = getenv("KRAKEN_AMD_GEMM_TILE")) {
-        if (t[0] == '1') big = false;
-        if (t[0] == '2') big = true;
-    }
+    if (env_switches().gemm_tile == 128) big = false;
+    if (env_switches().gemm_tile == 256) big = true;
     const bool dtl = big && gemm_dtl_supported(g) &&
                      (g.a_local == nullptr || (int64_t)256 * g.lda_local * 2 < 0x7fffffffLL);
     // The 128x128 kernel addresses a tile's operand panels with 32-bit byte offsets from the
@@ -631,7 +626,7 @@ static int gemm_reduce(const void* A, int64_t lda_m, int64_t lda_k, const void* 
     // KRAKEN_AMD_GEMM_PEERS=epilogue keeps the peers' partial sums out of the matrix cores
     // (they are then added in the epilogue, where a non-finite value stays in its element)
     g.peers_on_mfma = 1;
-    if (const char* t = getenv("KRAKEN_AMD_GEMM_PEERS")) g.peers_on_mfma = t[0] == 'e' ? 0 : t[0] == 'f' ? 2 : t[0] == 'l' ? 3 : 1;
+    if (env_switches().gemm_peers >= 0) g.peers_on_mfma = env_switches().gemm_peers;
     // MFMA block shape of the 256x256 kernel's k loop: 16x16x32 draws less power per flop than
     // 32x32x16 and the chip is power-limited (5-10 % faster with warm operands; results agree to fp32 rounding).  It
     // has no form that adds the peers on the matrix cores: its tiles add them in the epilogue,
@@ -639,7 +634,7 @@ static int gemm_reduce(const void* A, int64_t lda_m, int64_t lda_k, const void* 
     // of 1024 rows: 367 -> 354 us) and much when every tile has peers (4096x8192x1024: 120 ->
     // 146 us), so reduce-heavy calls keep 32x32x16.  KRAKEN_AMD_GEMM_MFMA=16|32 overrides.
     g.mi16 = !(n_peers > 0 && band_rows * 2 >= M);
-    if (const char* t = getenv("KRAKEN_AMD_GEMM_MFMA")) g.mi16 = t[0] == '1';
+    if (env_switches().gemm_mfma > 0) g.mi16 = env_switches().gemm_mfma == 16;
     const int bm = dtl ? 256 : 128, bn = bm;
     g.tiles_m = (int)((M + bm - 1) / bm);
     g.tiles_n = (int)((N + bn - 1) / bn);
@@ -659,10 +654,7 @@ static int gemm_reduce(const void* A, int64_t lda_m, int64_t lda_k, const void* 
     // band in the order of the destinations, and a band is complete once all eight have passed it
     // (with wide groups every band would only be complete when the last group is).
     if (g.progress != nullptr || g.band_counter != nullptr) g.group_n = (g.tiles_n + kXcds - 1) / kXcds;
-    if (const char* t = getenv("KRAKEN_AMD_GEMM_GROUP")) {
-        const int v = atoi(t);
-        if (v >= 1 && v <= 64) g.group_n = v;
-    }
+    if (const int v = env_switches().gemm_group; v >= 1 && v <= 64) g.group_n = v;
     // Split K loop (128x128 kernel, workspace given): with few tiles most CUs would idle, so S
     // workgroups share a tile's K loop and meet in the workspace.
     g.k_splits = 1;
@@ -778,10 +770,10 @@ extern "C" int kr_gemm_producer_bf16(const void* A, int64_t lda_m, int64_t lda_k
 extern "C" int64_t kr_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K) {
     if (M <= 0 || N <= 0 || K <= 0) return 0;
     // the large-tile kernel (same rule as the launch; strides are not known here)
-    const char* force_tile = getenv("KRAKEN_AMD_GEMM_TILE");
+    const int force_tile = env_switches().gemm_tile;
     bool big = ((M + 255) / 256) * ((N + 255) / 256) > 128 && K >= 256;
-    if (force_tile != nullptr && force_tile[0] == '1') big = false;
-    if (force_tile != nullptr && force_tile[0] == '2') big = true;
+    if (force_tile == 128) big = false;
+    if (force_tile == 256) big = true;
     if (big && K % 64 == 0 && K >= 64) {
         if (M % 256 != 0 || N % 256 != 0) return 0;
         int tail, ts;
@@ -792,7 +784,7 @@ extern "C" int64_t kr_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K) {
     const int S = split_k_factor(tiles, K);
     int64_t bytes = S > 1 ? split_k_workspace_bytes(M, N, S) : 0;
     // the layout of B is not known here: enough for either kernel
-    if (force_tile == nullptr && (whole_launch_split_pays(M, N, K, true, true) || whole_launch_split_pays(M, N, K, false, true))) {
+    if (force_tile < 0 && (whole_launch_split_pays(M, N, K, true, true) || whole_launch_split_pays(M, N, K, false, true))) {
         int tail, ts;
         tail_split_plan((M / 256) * (N / 256), K, &tail, &ts);
         if (tail > 0) bytes = std::max(bytes, gemm_dtl_tail_workspace_bytes(tail, ts));

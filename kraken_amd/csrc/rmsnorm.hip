@@ -7,8 +7,6 @@
 // of squares is reduced inside each wavefront with DPP lane permutes, then
 // across the wavefronts of the workgroup through a few words of LDS that every
 // wavefront re-reads and sums in the same way, so all threads hold the same rstd.
-#include <stdlib.h>
-
 #include "common.h"
 
 namespace kr {
@@ -157,6 +155,145 @@ __global__ __launch_bounds__(kMaxThreads) void reduce_rmsnorm_kernel(
     }
 }
 
+// ---- few long rows: one row on many compute units --------------------------------------------
+// One compute unit takes in about 55 GB/s, so a workgroup that owns a row of W * D * 2 bytes
+// needs W * D * 2 / 55e9 s however few rows there are (16 rows of 8 x 8192: 2.4 us of a 4.9 us
+// kernel on 16 of 256 compute units).  Here a row is cut into pieces of 64 vectors, one
+// wavefront (its own workgroup, any compute unit) each.  The wavefronts of a row meet in a
+// block of the caller's workspace: wavefront i stores {tag, its partial sum of squares} to slot i
+// with one 8-byte store, polls the row's slots until all carry the tag, and adds the partial sums
+// in slot order -- every wavefront of the row forms the same total in the same order, and the
+// result does not depend on who arrives when.  The tag is the row's generation + 1, read from the
+// block at the start of the kernel; wavefront 0 stores it back as the new generation once it has
+// seen every slot carry it (by then every wavefront of the row has read the old one).  No
+// read-modify-write, no reset, nothing to clear between calls: a slot left by an earlier call
+// carries a tag at or below the generation and never matches.  The accesses are relaxed atomics at
+// agent scope (they are served by the memory side, about 1 us a round trip, which is the price
+// of the exchange).  All wavefronts of a row are resident together (the grid is at most
+// kSplitMaxWaves one-wave workgroups, dispatched in order), so the poll ends; it is bounded all
+// the same and falls through after kSplitSpinLimit polls.
+constexpr int kSplitSlots = 64;                       // wavefronts per row at most -> D <= 32768
+constexpr int kSplitMaxRows = 64;
+constexpr int kSplitMaxWaves = 1024;
+constexpr int kSplitBlockWords = 16 + kSplitSlots;    // 8-byte words per row: generation (+ padding to 128 B), slots
+constexpr int64_t kSplitWorkspaceBytes = (int64_t)kSplitMaxRows * kSplitBlockWords * 8;
+constexpr int kSplitSpinLimit = 1 << 22;
+
+template <class SRC, int WT, int BIAS>
+__global__ __launch_bounds__(kWave) void reduce_rmsnorm_split_kernel(
+    const SRC src, int d_vec, int nw,
+    const u32x4* __restrict__ bias, const u32x4* __restrict__ wgt, float eps, float inv_d,
+    u32x4* __restrict__ y, uint64_t* __restrict__ ws) {
+    const int row = blockIdx.x / nw;
+    const int piece = blockIdx.x - row * nw;
+    const int lane = threadIdx.x;
+    const int c = piece * kWave + lane;
+    const int cc = min(c, d_vec - 1);
+    const int64_t row_v = (int64_t)row * d_vec;
+    uint64_t* block = ws + (int64_t)row * kSplitBlockWords;
+    uint64_t* slots = block + 16;
+
+    // every load of the wavefront is issued before the first is used
+    u32x4 x[WT];
+#pragma unroll
+    for (int r = 0; r < WT; ++r) x[r] = ld_stream(src.at(r) + row_v + cc);
+    u32x4 bv = {0, 0, 0, 0};
+    if (BIAS == kRowFullBias) bv = ld_stream(bias + row_v + cc);
+    else if (BIAS == kRowVecBias) bv = bias[cc];
+    const u32x4 wv = wgt[cc];
+    const uint32_t tag = (uint32_t)__hip_atomic_load(block, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) + 1u;
+
+    float s[8];
+    if (BIAS == kRowNoBias) zero8(s);
+    else unpack8(bv, s);
+#pragma unroll
+    for (int r = 0; r < WT; ++r) add8(x[r], s);
+    float ss = 0.0f;
+    if (c < d_vec) {
+#pragma unroll
+        for (int j = 0; j < 8; ++j) ss += s[j] * s[j];
+    }
+    ss = wave_sum(ss);
+
+    if (lane == 0)
+        __hip_atomic_store(slots + piece, ((uint64_t)tag << 32) | __builtin_bit_cast(uint32_t, ss), __ATOMIC_RELAXED,
+                           __HIP_MEMORY_SCOPE_AGENT);
+    uint64_t v = (uint64_t)tag << 32;
+    for (int spin = 0; spin < kSplitSpinLimit; ++spin) {
+        if (lane < nw) v = __hip_atomic_load(slots + lane, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (__all((uint32_t)(v >> 32) == tag)) break;
+        __builtin_amdgcn_s_sleep(1);
+    }
+    if (piece == 0 && lane == 0)
+        __hip_atomic_store(block, (uint64_t)tag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    float total = 0.0f;
+    const int part = (int)(uint32_t)v;
+    for (int k = 0; k < nw; ++k) total += __builtin_bit_cast(float, __builtin_amdgcn_readlane(part, k));
+    const float rstd = __builtin_amdgcn_rsqf(total * inv_d + eps);
+
+    if (c < d_vec) {
+        float wf[8], o[8];
+        unpack8(wv, wf);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) o[j] = (s[j] * rstd) * wf[j];
+        st_stream(y + row_v + c, pack8(o));
+    }
+}
+
+// Whether a call takes the split kernel (given a workspace).  Measured against one workgroup per
+// row with W = 8, inputs from HBM, rows = 1..64: D = 8192 wins up to 32 rows (1 row 4.0 -> 3.4 us,
+// 16 rows 5.0 -> 4.0 us, 32 rows 5.1 -> 5.0 us; 64 rows lose, 5.4 -> 6.4 us), D = 16384 up to 32 rows
+// (7.7 -> 6.0 us at 16), D = 32768 up to 16 rows (13.3 -> 9.4 us); D = 5120 is level and D <= 4096
+// loses 0.1 - 0.8 us: the exchange costs about 1.2 us, which a row of less than ~96 KiB does not
+// win back.
+static bool row_split_pays(int W, int64_t rows, int64_t D) {
+    if (!(W == 1 || W == 2 || W == 4 || W == 8)) return false;
+    const int64_t d_vec = D / 8;
+    const int64_t nw = (d_vec + kWave - 1) / kWave;
+    if (rows < 1 || rows > kSplitMaxRows || nw < 2 || nw > kSplitSlots || rows * nw > kSplitMaxWaves) return false;
+    if (env_switches().row_split >= 0) return env_switches().row_split != 0;
+    const int64_t row_bytes = (int64_t)W * D * 2;
+    return row_bytes >= 96 * 1024 && rows * nw <= (row_bytes >= 256 * 1024 ? 1024 : 512);
+}
+
+template <class SRC, int WT>
+static hipError_t launch_split2(int mode, dim3 grid, hipStream_t st, const SRC& tab, int d_vec, int nw,
+                                const u32x4* bias, const u32x4* wgt, float eps, float inv_d, u32x4* y, uint64_t* ws) {
+    switch (mode) {
+        case kRowNoBias:
+            hipLaunchKernelGGL((reduce_rmsnorm_split_kernel<SRC, WT, kRowNoBias>), grid, dim3(kWave), 0, st, tab, d_vec,
+                               nw, bias, wgt, eps, inv_d, y, ws);
+            break;
+        case kRowFullBias:
+            hipLaunchKernelGGL((reduce_rmsnorm_split_kernel<SRC, WT, kRowFullBias>), grid, dim3(kWave), 0, st, tab, d_vec,
+                               nw, bias, wgt, eps, inv_d, y, ws);
+            break;
+        default:
+            hipLaunchKernelGGL((reduce_rmsnorm_split_kernel<SRC, WT, kRowVecBias>), grid, dim3(kWave), 0, st, tab, d_vec,
+                               nw, bias, wgt, eps, inv_d, y, ws);
+            break;
+    }
+    return hipGetLastError();
+}
+
+template <class SRC>
+static int launch_split(const SRC& tab, int W, int64_t rows, int64_t D, const void* bias, int mode, const void* w,
+                        float eps, void* y, void* workspace, void* stream) {
+    const int d_vec = (int)(D / 8);
+    const int nw = (d_vec + kWave - 1) / kWave;
+    const dim3 grid((unsigned)(rows * nw));
+    const hipStream_t st = (hipStream_t)stream;
+    const u32x4* bp = (const u32x4*)bias;
+    const u32x4* wp = (const u32x4*)w;
+    const float inv_d = 1.0f / (float)D;
+    switch (W) {
+        case 1: return (int)launch_split2<SRC, 1>(mode, grid, st, tab, d_vec, nw, bp, wp, eps, inv_d, (u32x4*)y, (uint64_t*)workspace);
+        case 2: return (int)launch_split2<SRC, 2>(mode, grid, st, tab, d_vec, nw, bp, wp, eps, inv_d, (u32x4*)y, (uint64_t*)workspace);
+        case 4: return (int)launch_split2<SRC, 4>(mode, grid, st, tab, d_vec, nw, bp, wp, eps, inv_d, (u32x4*)y, (uint64_t*)workspace);
+        default: return (int)launch_split2<SRC, 8>(mode, grid, st, tab, d_vec, nw, bp, wp, eps, inv_d, (u32x4*)y, (uint64_t*)workspace);
+    }
+}
+
 template <class SRC, int VPT, int WT, bool LAT>
 static hipError_t launch_row2(int mode, dim3 grid, dim3 block, hipStream_t st, const SRC& tab, int W,
                               int d_vec, const u32x4* bias, const u32x4* wgt, float eps,
@@ -200,10 +337,8 @@ static void row_geometry(int d_vec, int* threads, int* vpt) {
     // with two; more wavefronts per row cost less than fewer loads in flight per thread)
     // KRAKEN_AMD_ROW_VPT=1|2|4|8 overrides the vectors per thread (tuning); ignored if a row
     // would need more than 1024 threads
-    if (const char* e = getenv("KRAKEN_AMD_ROW_VPT")) {
-        const int o = atoi(e);
-        if ((o == 1 || o == 2 || o == 4 || o == 8) && (int64_t)o * kMaxThreads >= d_vec) v = o;
-    }
+    if (const int o = env_switches().row_vpt; (o == 1 || o == 2 || o == 4 || o == 8) && (int64_t)o * kMaxThreads >= d_vec)
+        v = o;
     int t = (d_vec + v - 1) / v;
     t = (t + kWave - 1) / kWave * kWave;
     *threads = t;
@@ -212,7 +347,10 @@ static void row_geometry(int d_vec, int* threads, int* vpt) {
 
 template <class SRC>
 static int launch_rows(const SRC& tab, int W, int64_t rows, int64_t D, const void* bias,
-                       int mode, const void* w, float eps, void* y, void* stream) {
+                       int mode, const void* w, float eps, void* y, void* stream,
+                       void* workspace = nullptr, int64_t workspace_bytes = 0) {
+    if (workspace != nullptr && workspace_bytes >= kSplitWorkspaceBytes && row_split_pays(W, rows, D))
+        return launch_split(tab, W, rows, D, bias, mode, w, eps, y, workspace, stream);
     int threads, vpt;
     const int d_vec = (int)(D / 8);
     row_geometry(d_vec, &threads, &vpt);
@@ -220,7 +358,7 @@ static int launch_rows(const SRC& tab, int W, int64_t rows, int64_t D, const voi
     // latency-first instantiation is 9 % faster at [256, 4096], 2.5 % at [16, 8192]; with many
     // rows it is level or up to 2 % slower (KRAKEN_AMD_ROW_LAT=0|1 overrides, for tuning)
     bool lat = rows <= kLatRows;
-    if (const char* e = getenv("KRAKEN_AMD_ROW_LAT")) lat = e[0] == '1';
+    if (env_switches().row_lat >= 0) lat = env_switches().row_lat == 1;
     const dim3 grid((unsigned)rows), block((unsigned)threads);
     const hipStream_t st = (hipStream_t)stream;
     const u32x4* bp = (const u32x4*)bias;
@@ -259,28 +397,47 @@ static int check_rows(int W, int64_t rows, int64_t D, const void* bias, const vo
     return KR_OK;
 }
 
-extern "C" int kr_reduce_rmsnorm_bf16(const void* stack, int W, int64_t slice_stride, int64_t rows, int64_t D,
-                                      const void* bias, int bias_is_vector, const void* w, float eps, void* y,
-                                      void* stream) {
+extern "C" int64_t kr_rmsnorm_workspace_bytes(int W, int64_t rows, int64_t D) {
+    if (D <= 0 || D % 8 != 0) return 0;
+    return row_split_pays(W, rows, D) ? kSplitWorkspaceBytes : 0;
+}
+
+extern "C" int kr_reduce_rmsnorm_ws_bf16(const void* stack, int W, int64_t slice_stride, int64_t rows, int64_t D,
+                                         const void* bias, int bias_is_vector, const void* w, float eps, void* y,
+                                         void* workspace, int64_t workspace_bytes, void* stream) {
     if (W >= 1 && W <= KR_MAX_WORLD && slice_stride < 0) return KR_ERR_BAD_DIM;
     int rc = check_rows(W, rows, D, bias, w, y);
     if (rc != KR_OK || rows == 0) return rc;
     if (stack == nullptr) return KR_ERR_NULL_POINTER;
-    if (!aligned16(stack) || slice_stride % 8 != 0) return KR_ERR_ALIGNMENT;
+    if (!aligned16(stack) || slice_stride % 8 != 0 || !aligned16(workspace)) return KR_ERR_ALIGNMENT;
     const int mode = bias == nullptr ? kRowNoBias : (bias_is_vector ? kRowVecBias : kRowFullBias);
     const StackedPeers src{(const u32x4*)stack, slice_stride / 8};
-    return launch_rows(src, W, rows, D, bias, mode, w, eps, y, stream);
+    return launch_rows(src, W, rows, D, bias, mode, w, eps, y, stream, workspace, workspace_bytes);
+}
+
+extern "C" int kr_reduce_rmsnorm_bf16(const void* stack, int W, int64_t slice_stride, int64_t rows, int64_t D,
+                                      const void* bias, int bias_is_vector, const void* w, float eps, void* y,
+                                      void* stream) {
+    return kr_reduce_rmsnorm_ws_bf16(stack, W, slice_stride, rows, D, bias, bias_is_vector, w, eps, y, nullptr, 0,
+                                     stream);
+}
+
+extern "C" int kr_reduce_rmsnorm_ptrs_ws_bf16(const void* const* bufs, int W, int64_t rows, int64_t D,
+                                              const void* bias, int bias_is_vector, const void* w, float eps,
+                                              void* y, void* workspace, int64_t workspace_bytes, void* stream) {
+    int rc = check_rows(W, rows, D, bias, w, y);
+    if (rc != KR_OK || rows == 0) return rc;
+    PeerTab tab;
+    if ((rc = peer_tab_from_ptrs(tab, bufs, W)) != KR_OK) return rc;
+    if (!aligned16(workspace)) return KR_ERR_ALIGNMENT;
+    const int mode = bias == nullptr ? kRowNoBias : (bias_is_vector ? kRowVecBias : kRowFullBias);
+    return launch_rows(tab, W, rows, D, bias, mode, w, eps, y, stream, workspace, workspace_bytes);
 }
 
 extern "C" int kr_reduce_rmsnorm_ptrs_bf16(const void* const* bufs, int W, int64_t rows, int64_t D,
                                            const void* bias, int bias_is_vector, const void* w, float eps,
                                            void* y, void* stream) {
-    int rc = check_rows(W, rows, D, bias, w, y);
-    if (rc != KR_OK || rows == 0) return rc;
-    PeerTab tab;
-    if ((rc = peer_tab_from_ptrs(tab, bufs, W)) != KR_OK) return rc;
-    const int mode = bias == nullptr ? kRowNoBias : (bias_is_vector ? kRowVecBias : kRowFullBias);
-    return launch_rows(tab, W, rows, D, bias, mode, w, eps, y, stream);
+    return kr_reduce_rmsnorm_ptrs_ws_bf16(bufs, W, rows, D, bias, bias_is_vector, w, eps, y, nullptr, 0, stream);
 }
 
 extern "C" int kr_rmsnorm_bf16(const void* x, const void* w, float eps, int64_t rows, int64_t D, void* y,

@@ -1,6 +1,35 @@
 // Version and error-text entry points of the C ABI.
 #include "common.h"
 
+#include <stdlib.h>
+
+namespace kr {
+static EnvSwitches read_env() {
+    EnvSwitches e;
+    auto num = [](const char* name) { const char* t = getenv(name); return t != nullptr && t[0] != 0 ? atoi(t) : -1; };
+    e.row_vpt = num("KRAKEN_AMD_ROW_VPT");
+    e.row_lat = num("KRAKEN_AMD_ROW_LAT");
+    e.row_split = num("KRAKEN_AMD_ROW_SPLIT");
+    const char* t = getenv("KRAKEN_AMD_GEMM_TILE");
+    e.gemm_tile = t == nullptr ? -1 : t[0] == '1' ? 128 : t[0] == '2' ? 256 : -1;
+    t = getenv("KRAKEN_AMD_GEMM_PEERS");
+    e.gemm_peers = t == nullptr ? -1 : t[0] == 'e' ? 0 : t[0] == 'f' ? 2 : t[0] == 'l' ? 3 : 1;
+    t = getenv("KRAKEN_AMD_GEMM_MFMA");
+    e.gemm_mfma = t == nullptr ? -1 : t[0] == '1' ? 16 : 32;
+    e.gemm_group = num("KRAKEN_AMD_GEMM_GROUP");
+    e.gemm_splitk = num("KRAKEN_AMD_GEMM_SPLITK");
+    e.gemm_tailsplit = num("KRAKEN_AMD_GEMM_TAILSPLIT");
+    return e;
+}
+static EnvSwitches& env_storage() {
+    static EnvSwitches e = read_env();
+    return e;
+}
+const EnvSwitches& env_switches() { return env_storage(); }
+}  // namespace kr
+
+extern "C" void kr_reload_env(void) { kr::env_storage() = kr::read_env(); }
+
 extern "C" int kr_version(void) { return 100; }  // 0.1.0
 
 extern "C" const char* kr_strerror(int code) {

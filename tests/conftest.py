@@ -46,3 +46,38 @@ def oracle_c():
 @pytest.fixture(scope="session")
 def dev():
     return torch.device("cuda:0")
+
+
+class _EnvAwareMonkeyPatch:
+    """pytest's monkeypatch, except that a change to a KRAKEN_AMD_* variable also makes the
+    library read its switches again (it reads the environment once per process)."""
+
+    def __init__(self, inner):
+        self._inner = inner
+
+    def __getattr__(self, name):
+        return getattr(self._inner, name)
+
+    @staticmethod
+    def _reload(name):
+        if name.startswith("KRAKEN_AMD_"):
+            from kraken_amd import _lib
+
+            _lib.reload_env()
+
+    def setenv(self, name, value, prepend=None):
+        self._inner.setenv(name, value, prepend)
+        self._reload(name)
+
+    def delenv(self, name, raising=True):
+        self._inner.delenv(name, raising)
+        self._reload(name)
+
+
+@pytest.fixture
+def monkeypatch(monkeypatch):
+    yield _EnvAwareMonkeyPatch(monkeypatch)
+    monkeypatch.undo()
+    from kraken_amd import _lib
+
+    _lib.reload_env()

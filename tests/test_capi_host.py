@@ -66,6 +66,27 @@ def test_rmsnorm_argument_errors(lib):
     assert g(FAKE, FAKE + 8, 1e-5, 4, 64, FAKE, None) == _lib.KR_ERR_ALIGNMENT
 
 
+def test_rmsnorm_workspace_entries(lib, monkeypatch):
+    """Which shapes the split-row kernel takes (a few long rows), and that the workspace forms
+    validate like the plain ones."""
+    q = lib.kr_rmsnorm_workspace_bytes
+    need = q(8, 16, 8192)
+    assert need > 0 and q(8, 1, 8192) == need and q(4, 16, 32768) == need
+    assert q(8, 256, 4096) == 0 and q(8, 16, 1024) == 0 and q(3, 16, 8192) == 0 and q(8, 128, 8192) == 0
+    assert q(8, 16, 8190) == 0 and q(8, 0, 8192) == 0 and q(8, 2, 65536) == 0
+    f = lib.kr_reduce_rmsnorm_ws_bf16
+    assert f(FAKE, 8, 8192 * 16, 16, 8192, None, 0, FAKE, 1e-5, FAKE, FAKE + 8, need, None) == _lib.KR_ERR_ALIGNMENT
+    assert f(FAKE, 8, 8192 * 16, 16, 8196, None, 0, FAKE, 1e-5, FAKE, FAKE, need, None) == _lib.KR_ERR_NUMEL_MOD8
+    assert f(None, 8, 8192 * 16, 16, 8192, None, 0, FAKE, 1e-5, FAKE, FAKE, need, None) == _lib.KR_ERR_NULL_POINTER
+    assert f(FAKE, 8, 8192 * 16, 0, 8192, None, 0, FAKE, 1e-5, FAKE, FAKE, need, None) == 0
+    g = lib.kr_reduce_rmsnorm_ptrs_ws_bf16
+    assert g(None, 8, 16, 8192, None, 0, FAKE, 1e-5, FAKE, FAKE, need, None) == _lib.KR_ERR_NULL_POINTER
+    monkeypatch.setenv("KRAKEN_AMD_ROW_SPLIT", "0")
+    assert q(8, 16, 8192) == 0
+    monkeypatch.setenv("KRAKEN_AMD_ROW_SPLIT", "1")
+    assert q(8, 64, 1024) == need and q(8, 65, 1024) == 0 and q(8, 1, 512) == 0   # 64 rows at most, two wavefronts at least
+
+
 def test_gemm_argument_errors(lib):
     f = lib.kr_gemm_reduce_bf16
 

@@ -133,3 +133,96 @@ def test_baseline_configs_1_and_3(dev, cfg):
     y2 = torch.empty_like(y)
     fused.one_shot_all_reduce_bias_rms_norm((stack * 2).to(dev), None, (bias * 2).to(dev), w.to(dev), y2, eps=1e-5)
     torch.testing.assert_close(y2.float().cpu(), y.float().cpu(), rtol=2 ** -7, atol=1e-5)
+
+
+# ---- a few long rows: one row spread over many compute units (split-row kernel) ----------------
+
+def _split_used(W, rows, D):
+    from kraken_amd import _lib
+    return _lib.load().kr_rmsnorm_workspace_bytes(W, rows, D) > 0
+
+
+@pytest.mark.parametrize("W,rows,D", [(8, 16, 8192), (8, 1, 8192), (8, 5, 16384), (4, 3, 32768), (8, 7, 8200),
+                                      (2, 3, 1024), (1, 2, 4096), (8, 64, 1024)])
+@pytest.mark.parametrize("bias_mode", ["none", "full", "vector"])
+def test_split_rows_match_the_oracle(dev, monkeypatch, W, rows, D, bias_mode):
+    """Forced on for every shape it can take: rows whose last wavefront is ragged (D = 8200),
+    two to 64 wavefronts per row, every W it is instantiated for, every bias form; stacked and
+    separate buffers give the same bits; against the one-workgroup kernel at most an ulp."""
+    monkeypatch.setenv("KRAKEN_AMD_ROW_SPLIT", "1")
+    assert _split_used(W, rows, D)
+    stack = orc.make_stack(W, (rows, D), seed0=11)
+    w = orc.randn_bf16((D,), 5, 0.02, 1.0)
+    bias = {"none": None, "full": orc.randn_bf16((rows, D), 7), "vector": orc.randn_bf16((D,), 7, 0.02)}[bias_mode]
+    bd = None if bias is None else bias.to(dev)
+    sd, wd = stack.to(dev), w.to(dev)
+    want = orc.reduce_bias_rms_norm(stack, bias, w, 1e-5)
+    y = torch.empty(rows, D, dtype=BF16, device=dev)
+    fused.one_shot_all_reduce_bias_rms_norm(sd, None, bd, wd, y, eps=1e-5)
+    torch.testing.assert_close(y.cpu(), want, **TOL)
+    assert_one_ulp(y, want)
+    y2 = torch.full_like(y, 3.0)
+    fused.one_shot_all_reduce_bias_rms_norm([sd[r].clone() for r in range(W)], None, bd, wd, y2, eps=1e-5)
+    assert torch.equal(y.view(torch.int16), y2.view(torch.int16))
+    monkeypatch.setenv("KRAKEN_AMD_ROW_SPLIT", "0")
+    assert not _split_used(W, rows, D)
+    y3 = torch.empty_like(y)
+    fused.one_shot_all_reduce_bias_rms_norm(sd, None, bd, wd, y3, eps=1e-5)
+    assert_one_ulp(y3, want)
+    assert (y3 == y).float().mean() > 0.99
+
+
+def test_split_rows_default_rule(dev):
+    """The decode shape of the benchmark takes the split kernel by default, the 256-row shape and
+    short rows do not."""
+    assert _split_used(8, 16, 8192) and _split_used(8, 1, 8192)
+    assert not _split_used(8, 256, 4096) and not _split_used(8, 16, 1024) and not _split_used(3, 16, 8192)
+
+
+def test_split_rows_share_one_workspace_across_shapes_and_calls(dev, monkeypatch):
+    """Calls of different shapes in a row on one stream share the stream's workspace, which is never
+    cleared in between: slots left by a wider call must not be taken for this call's."""
+    monkeypatch.setenv("KRAKEN_AMD_ROW_SPLIT", "1")
+    cases = []
+    for i, (W, rows, D) in enumerate([(8, 16, 8192), (8, 3, 32768), (4, 64, 1024), (8, 1, 8192), (2, 16, 16384)]):
+        stack = orc.make_stack(W, (rows, D), seed0=50 + i)
+        bias, w = orc.make_bias_weight(D, 60 + i)
+        cases.append((stack.to(dev), bias.to(dev), w.to(dev), torch.empty(rows, D, dtype=BF16, device=dev),
+                      orc.reduce_bias_rms_norm(stack, bias, w, 1e-5)))
+    for rep in range(4):
+        order = cases if rep % 2 == 0 else cases[::-1]
+        for (sd, bd, wd, y, want) in order:
+            y.zero_()
+            fused.one_shot_all_reduce_bias_rms_norm(sd, None, bd, wd, y, eps=1e-5)
+        torch.cuda.synchronize()
+        for (sd, bd, wd, y, want) in cases:
+            assert_one_ulp(y, want)
+
+
+def test_split_rows_replay_from_a_graph(dev):
+    """Captured once, replayed with eager calls (which advance the rows' generations) in between:
+    every replay gives the eager bits."""
+    W, rows, D = 8, 16, 8192
+    assert _split_used(W, rows, D)
+    stack = orc.make_stack(W, (rows, D), seed0=42).to(dev)
+    bias, w = (t.to(dev) for t in orc.make_bias_weight(D, 42))
+    y = torch.empty(rows, D, dtype=BF16, device=dev)
+    fused.one_shot_all_reduce_bias_rms_norm(stack, None, bias, w, y)
+    eager = y.clone()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    g = torch.cuda.CUDAGraph()
+    yg = torch.empty_like(y)
+    with torch.cuda.stream(side):
+        fused.one_shot_all_reduce_bias_rms_norm(stack, None, bias, w, yg)   # the stream's workspace exists
+        side.synchronize()
+        with torch.cuda.graph(g, stream=side):
+            for _ in range(3):
+                fused.one_shot_all_reduce_bias_rms_norm(stack, None, bias, w, yg)
+    for rep in range(3):
+        yg.zero_()
+        fused.one_shot_all_reduce_bias_rms_norm(stack, None, bias, w, y)       # eager work between the replays
+        torch.cuda.synchronize()
+        g.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(yg, eager)
