@@ -14,9 +14,12 @@ checked against the CPU oracle before it is timed.
 
 Timing: W untimed warm-up steps, then exactly K steps between two device
 synchronisations; events recorded on the launch stream around the same K
-steps give the average kernel duration used for the roofline figure.  The
-input set is rotated every step (several sets, together larger than the
-256 MB last-level cache), so no step finds its input cached.
+steps give the average kernel duration used for the roofline figure.  Every
+workload rotates several complete operand sets (inputs, peers and outputs,
+the GEMM operands A and B included), together larger than the 256 MB
+last-level cache, so no step finds its operands cached.  Each entry states
+the target the benchmark definition gives for it (a fraction of the HBM or
+bf16 matrix-core peak) and whether the measured figure meets it.
 """
 from __future__ import annotations
 
@@ -34,12 +37,29 @@ HBM_PEAK_GBS = 8000.0            # MI355X HBM3E
 MFMA_BF16_PEAK_TFLOPS = 2500.0   # MI355X dense bf16
 W = 8
 
-# HBM bytes per launch of the dominant kernel, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of
-# `bench.py --only --no-cpu`, each counter scaled by what it reads for a plain 256 MiB device copy
-# (`bench.py --calibrate-copy`).  bench.py cannot read hardware counters itself; the figures and the
-# commands behind them are kept as text under profiles/.
+# HBM-side bytes per launch of the dominant kernel (L2 fills + write-backs), from rocprofv3 --pmc
+# FETCH_SIZE / WRITE_SIZE runs of `bench.py --only --no-cpu --workload <key>`, each counter scaled by
+# what it reads for a plain 256 MiB device copy (`bench.py --calibrate-copy`).  bench.py cannot read
+# hardware counters itself; the figures and the commands behind them are kept as text under
+# profiles/ (one file per kernel and workload).  None: not measured.
 MEASURED_TRAFFIC = {
     "one_shot_reduce_w8_4096x4096": 302054820,
+}
+
+# Targets of the benchmark definition: fraction of the binding roof.  The W = 8 reduce(+bias+RMSNorm)
+# paths: 75 % of peak HBM bandwidth; the GEMM + reduce paths at the Llama-70B TP8 shard shapes: 60 %
+# of the dense bf16 matrix-core peak.  The decode shape is latency-bound (reported in microseconds
+# beside the launch floor) and the fused GEMM + all-reduce is HBM-bound (122 flop/B: its matrix-core
+# fraction cannot exceed 39 %), so neither has a target of its own.
+TARGETS = {
+    "one_shot_reduce_w8_4096x4096": ("hbm", 0.75),
+    "two_shot_share_w8_512x4096": ("hbm", 0.75),
+    "reduce_bias_rmsnorm_w8_256x4096": ("hbm", 0.75),
+    "reduce_bias_rmsnorm_w8_16x8192_decode": (None, None),
+    "reduce_bias_rmsnorm_w8_16384x4096_large": ("hbm", 0.75),
+    "gemm_reduce_scatter_8192x8192x3584_w8": ("mfma", 0.60),
+    "gemm_all_reduce_4096x8192x1024_w8": (None, None),
+    "all_gather_matmul_8192x3584x8192_w8": ("mfma", 0.60),
 }
 
 
@@ -211,6 +231,7 @@ class GemmReduceScatter(Workload):
     bound = "mfma"
     M, N, K = 8192, 8192, 3584
     cpu_repeats = 3
+    nsets = 3   # 3 x 386 MB of A, B, peers and outputs in rotation: every step's operands come from HBM
 
     def __init__(self):
         self.flops = 2 * self.M * self.N * self.K
@@ -224,14 +245,17 @@ class GemmReduceScatter(Workload):
         self.ha = orc.randn_bf16((self.M, self.K), 42)
         self.hb = orc.randn_bf16((self.K, self.N), 43, 0.02)
         self.hp = torch.stack([orc.randn_bf16((self.M // W, self.N), 100 + j) for j in range(W - 1)])
-        self.a, self.b, self.p = self.ha.to(dev), self.hb.to(dev), self.hp.to(dev)
-        self.c = torch.empty(self.M, self.N, dtype=torch.bfloat16, device=dev)
+        self.a = [self.ha.to(dev)] + _rand_sets((self.M, self.K), self.nsets - 1, dev, seed=1)
+        self.b = [self.hb.to(dev)] + _rand_sets((self.K, self.N), self.nsets - 1, dev, std=0.02, seed=2)
+        self.p = [self.hp.to(dev)] + _rand_sets((W - 1, self.M // W, self.N), self.nsets - 1, dev, seed=3)
+        self.c = [torch.empty(self.M, self.N, dtype=torch.bfloat16, device=dev) for _ in range(self.nsets)]
         self.out = None
 
     def step(self, i):
         from kraken_amd import fused
 
-        self.out = fused.gemm_reduce_scatter(self.a, self.b, peers=self.p, rank=self.rank, c_scratch=self.c)
+        j = i % self.nsets
+        self.out = fused.gemm_reduce_scatter(self.a[j], self.b[j], peers=self.p[j], rank=self.rank, c_scratch=self.c[j])
 
     def check(self):
         import torch
@@ -242,7 +266,7 @@ class GemmReduceScatter(Workload):
         want = self.ha[r0 + pick].float() @ self.hb.float() + self.hp[:, pick].float().sum(0)
         torch.testing.assert_close(self.out.cpu()[pick].float(), want.to(torch.bfloat16).float(), rtol=2e-2, atol=2e-2)
         other = torch.tensor([0, 4096, 8191])   # rows outside the band of rank 3
-        torch.testing.assert_close(self.c.cpu()[other].float(),
+        torch.testing.assert_close(self.c[0].cpu()[other].float(),
                                    (self.ha[other].float() @ self.hb.float()).to(torch.bfloat16).float(),
                                    rtol=2e-2, atol=2e-2)
         return "sampled rows within rtol=atol=2e-2 of the oracle"
@@ -253,7 +277,8 @@ class GemmReduceScatter(Workload):
         return orc.gemm_reduce_scatter(self.ha, self.hb, self.hp, self.rank, W)
 
     def describe(self):
-        return {"M": self.M, "N": self.N, "K": self.K, "peers": [7, 1024, self.N], "kernel": "gemm_dtl16_kernel"}
+        return {"M": self.M, "N": self.N, "K": self.K, "peers": [7, 1024, self.N], "kernel": "gemm_dtl16_kernel",
+                "operand_sets": self.nsets}
 
 
 class GemmAllReduce(Workload):
@@ -276,7 +301,9 @@ class GemmAllReduce(Workload):
         self.hb = orc.randn_bf16((self.K, self.N), 43, 0.02)
         self.hbias = orc.randn_bf16((self.N,), 42, 0.02)
         self.hp = torch.stack([orc.randn_bf16((self.M, self.N), 100 + j) for j in range(W - 1)])
-        self.a, self.b, self.bias = self.ha.to(dev), self.hb.to(dev), self.hbias.to(dev)
+        self.bias = self.hbias.to(dev)
+        self.a = [self.ha.to(dev)] + _rand_sets((self.M, self.K), self.nsets - 1, dev, seed=1)
+        self.b = [self.hb.to(dev)] + _rand_sets((self.K, self.N), self.nsets - 1, dev, std=0.02, seed=2)
         self.psets = [self.hp.to(dev)] + _rand_sets((W - 1, self.M, self.N), self.nsets - 1, dev)
         self.out = None
 
@@ -284,7 +311,8 @@ class GemmAllReduce(Workload):
         import torch
         from kraken_amd import fused
 
-        self.out = fused.gemm_one_shot_all_reduce_fused(self.a, self.b, peers=self.psets[i % self.nsets],
+        j = i % self.nsets
+        self.out = fused.gemm_one_shot_all_reduce_fused(self.a[j], self.b[j], peers=self.psets[j],
                                                         bias=self.bias, out_dtype=torch.bfloat16)
 
     def check(self):
@@ -304,7 +332,7 @@ class GemmAllReduce(Workload):
 
     def describe(self):
         return {"M": self.M, "N": self.N, "K": self.K, "peers": [7, self.M, self.N], "bias": [self.N],
-                "kernel": "gemm_dtl_kernel"}
+                "kernel": "gemm_dtl_kernel", "operand_sets": self.nsets}
 
 
 class AllGatherMatmul(Workload):
@@ -313,6 +341,7 @@ class AllGatherMatmul(Workload):
     bound = "mfma"
     m, K, N = 1024, 8192, 3584
     cpu_repeats = 3
+    nsets = 3   # 3 x 252 MB of A shards, B and C in rotation: every step's operands come from HBM
 
     def __init__(self):
         self.flops = 2 * W * self.m * self.N * self.K
@@ -323,13 +352,16 @@ class AllGatherMatmul(Workload):
 
         self.hs = orc.make_stack(W, (self.m, self.K), seed0=42)
         self.hbT = orc.randn_bf16((self.N, self.K), 43, 0.02)
-        self.s, self.bT = self.hs.to(dev), self.hbT.to(dev)
-        self.c = None
+        self.s = [self.hs.to(dev)] + _rand_sets((W, self.m, self.K), self.nsets - 1, dev, seed=1)
+        self.bT = [self.hbT.to(dev)] + _rand_sets((self.N, self.K), self.nsets - 1, dev, std=0.02, seed=2)
+        self.c = [None] * self.nsets
 
     def step(self, i):
         from kraken_amd import fused
 
-        _, self.c = fused.all_gather_matmul(self.s, self.bT.T, rank=3)
+        j = i % self.nsets
+        self.c[j] = None                         # (the allocator hands this set's own block back)
+        _, self.c[j] = fused.all_gather_matmul(self.s[j], self.bT[j].T, rank=3)
 
     def check(self):
         import torch
@@ -337,7 +369,7 @@ class AllGatherMatmul(Workload):
         self.step(0)
         pick = torch.tensor([0, 1023, 3072, 8191])
         want = self.hs.reshape(-1, self.K)[pick].float() @ self.hbT.T.float()
-        torch.testing.assert_close(self.c.cpu()[pick].float(), want.to(torch.bfloat16).float(), rtol=2e-2, atol=2e-2)
+        torch.testing.assert_close(self.c[0].cpu()[pick].float(), want.to(torch.bfloat16).float(), rtol=2e-2, atol=2e-2)
         return "sampled rows within rtol=atol=2e-2 of the oracle"
 
     def cpu_step(self):
@@ -346,7 +378,8 @@ class AllGatherMatmul(Workload):
         return orc.all_gather_matmul(self.hs, self.hbT.T)
 
     def describe(self):
-        return {"W": W, "m": self.m, "K": self.K, "N": self.N, "b_layout": "b.T contiguous", "kernel": "gemm_dtl16_kernel"}
+        return {"W": W, "m": self.m, "K": self.K, "N": self.N, "b_layout": "b.T contiguous", "kernel": "gemm_dtl16_kernel",
+                "operand_sets": self.nsets}
 
 
 def make_workloads():
@@ -436,6 +469,33 @@ def time_cpu(wl, budget_s=12.0):
     return times[len(times) // 2], len(times)
 
 
+def launch_floor_us(steps=200):
+    """Microseconds per launch of a kernel that does nothing but one 4-byte store, replayed from a
+    HIP graph like the microsecond workloads: what any kernel costs here before it moves a byte."""
+    import torch
+    from kraken_amd import _lib
+
+    lib = _lib.load()
+    word = torch.zeros(1, dtype=torch.int32, device="cuda")
+
+    class _Floor:
+        use_graph = True
+
+        def step(self, i):
+            lib.kr_stream_write_value32(word.data_ptr(), 1, torch.cuda.current_stream().cuda_stream)
+
+    return time_gpu_graph(_Floor(), steps, 5)[1] * 1e3
+
+
+def target_of(name, rec):
+    """The benchmark definition's target for a workload and whether the measured figure meets it."""
+    roof, frac = TARGETS.get(name, (None, None))
+    if roof is None:
+        return {"target": None, "meets_target": None}
+    got = rec["mfma_frac"] if roof == "mfma" else rec["hbm_frac"]
+    return {"target": {"roof": roof, "frac": frac}, "meets_target": bool(got >= frac)}
+
+
 def measure(wl, steps, warmup, dev, with_cpu, cpu_budget):
     import torch
 
@@ -451,11 +511,15 @@ def measure(wl, steps, warmup, dev, with_cpu, cpu_budget):
         "hbm_frac": wl.bytes / (ev_ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
         "bound": wl.bound,
         "timing": "hip graph replay" if getattr(wl, "use_graph", False) else "eager launches",
+        "algorithmic_bytes": wl.bytes,
+        "traffic": MEASURED_TRAFFIC.get(wl.name),
         **wl.describe(),
     }
     if wl.flops:
         rec["tflops"] = wl.flops / (ev_ms * 1e-3) / 1e12
         rec["mfma_frac"] = rec["tflops"] / MFMA_BF16_PEAK_TFLOPS
+        rec["algorithmic_flops"] = wl.flops
+    rec.update(target_of(wl.name, rec))
     if with_cpu:
         cpu_s, n = time_cpu(wl, cpu_budget)
         rec["cpu_ms"] = cpu_s * 1e3
@@ -558,6 +622,8 @@ def main() -> None:
             "algorithmic_bytes": main_wl.bytes,
             "algorithmic_flops": main_wl.flops,
         },
+        "target": rec["target"],
+        "meets_target": rec["meets_target"],
     }
     if not args.no_cpu:
         line["cpu_baseline"] = {
@@ -591,6 +657,11 @@ def main() -> None:
             del wl
             torch.cuda.empty_cache()
         line["configs"] = others
+        # what a launch costs before it moves a byte, in the protocol of the microsecond workloads
+        # (the decode shape and the 256-row shape are reported beside it)
+        line["launch_floor_us"] = launch_floor_us()
+        met = [r.get("meets_target") for r in others] + [line["meets_target"]]
+        line["targets_met"] = f"{sum(1 for m in met if m)} of {sum(1 for m in met if m is not None)} stated targets"
     print(json.dumps(line))
 
 
