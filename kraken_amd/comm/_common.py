@@ -112,20 +112,41 @@ def check_stack(stacked: torch.Tensor | Sequence[torch.Tensor]) -> PeerBuffers:
     return PeerBuffers(stacked)
 
 
-def stage_input(peers: PeerBuffers, input_tensor: torch.Tensor | None, rank: int) -> None:
-    """Copy ``input_tensor`` into the buffer of rank ``rank``.
+def stage_input(peers: PeerBuffers, input_tensor: torch.Tensor | None, rank: int, stage: bool = False) -> PeerBuffers:
+    """Make ``input_tensor`` the source of rank ``rank`` and return the buffers to reduce.
 
-    Stands in for the copy-in stage of the reference kernels
-    (``kraken/fused/one_shot_all_reduce_bias.py:56-65``).  Skipped when the
-    tensor already is (a prefix of) that buffer.
+    The reference kernels first copy the input into this rank's symmetric buffer, where the
+    peers read it (``kraken/fused/one_shot_all_reduce_bias.py:56-65``,
+    ``one_shot_all_reduce_bias_rms_norm.py:57-61``).  On one GPU nobody else reads that buffer, so
+    by default the input is read in place: the returned buffers are the W sources as a pointer
+    table whose entry ``rank`` is the input itself -- no copy, no extra launch, the same bits.
+    ``stage=True`` keeps the side effect for callers who want the buffer to hold the input
+    afterwards: one device copy into the buffer in front of the kernel.  An input that is not
+    contiguous or not 16-byte aligned is always copied.
     """
     if input_tensor is None:
-        return
+        return peers
     n = input_tensor.numel()
     dst = peers.slice(rank).reshape(-1)[:n]
     if dst.data_ptr() == input_tensor.data_ptr():
-        return
-    dst.copy_(input_tensor.reshape(-1))
+        return peers
+    if stage or not input_tensor.is_contiguous() or input_tensor.data_ptr() % 16 != 0:
+        dst.copy_(input_tensor.reshape(-1))
+        return peers
+    sources = [peers.slice(r).reshape(-1) for r in range(peers.W)]
+    sources[rank] = input_tensor.reshape(-1)
+    return _Sources(sources, peers.cap)
+
+
+class _Sources(PeerBuffers):
+    """W flat sources of possibly different lengths (each at least as long as the message)."""
+
+    def __init__(self, sources: Sequence[torch.Tensor], cap: int):
+        self.W = len(sources)
+        self.cap = cap
+        self.stride = None
+        self.stacked = None
+        self.tensors = list(sources)
 
 
 def bias_args(bias: torch.Tensor | None, numel: int, D: int) -> tuple[int | None, int]:

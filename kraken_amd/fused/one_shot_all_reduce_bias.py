@@ -17,6 +17,7 @@ def one_shot_all_reduce_bias(
     group=None,
     *,
     rank: int = 0,
+    stage: bool = False,
 ) -> None:
     """``output = bias + sum over the W slices`` (bias first, then slices 0..W-1, fp32).
 
@@ -27,9 +28,11 @@ def one_shot_all_reduce_bias(
     symmetric-memory buffers, or a list of W separate tensors; each slice may be larger than the input, only its
     first ``output.numel()`` elements are used (the reference rendezvouses on a
     buffer larger than the message as well, ``test/test_allreduce_bias.py:57-62``).
-    ``input_tensor``, if given, is first copied into slice ``rank`` — the
-    reference's copy-in (``:56-65``); pass ``None`` when the stack is already
-    staged.  ``bias`` has the shape of the input (as the reference passes it)
+    ``input_tensor``, if given, is rank ``rank``'s contribution in place of slice ``rank``:
+    it is read where it lies, inside the one kernel (the reference's fused copy-in ``:56-65``
+    exists so that the peers can read it; here nobody else does); ``stage=True`` also copies it
+    into slice ``rank`` first, for callers who want that side effect.  Pass ``None`` when the
+    stack is already staged.  ``bias`` has the shape of the input (as the reference passes it)
     or is a vector over the last dimension, or ``None`` (plain sum, ``:80-84``).
     ``max_num_blocks``, ``BLOCK_SIZE`` and ``group`` are accepted and ignored.
     """
@@ -47,6 +50,6 @@ def one_shot_all_reduce_bias(
     D = ref.shape[-1] if ref.dim() >= 1 else numel
     bias_ptr, bias_numel = bias_args(bias, numel, D)
     dev = _lib.require_device(*peers.tensors, input_tensor, bias, output)
-    stage_input(peers, input_tensor, rank)
+    peers = stage_input(peers, input_tensor, rank, stage)
     rc = peers.reduce(0, numel, bias_ptr, bias_numel, D, 1, output.data_ptr(), _lib.current_stream(dev))
     _lib.check(rc, "one_shot_all_reduce_bias")

@@ -9,7 +9,7 @@ from .. import _lib
 from ..comm._common import check_stack, stage_input
 
 
-def _launch_reduce_rms_norm(name, symm_mem_input, x, bias, w, y, eps, rank):
+def _launch_reduce_rms_norm(name, symm_mem_input, x, bias, w, y, eps, rank, stage=False):
     D = y.shape[-1]
     if x is not None:
         assert y.shape == x.shape
@@ -32,7 +32,7 @@ def _launch_reduce_rms_norm(name, symm_mem_input, x, bias, w, y, eps, rank):
         assert bias.numel() in (rows * D, D), "bias must have the shape of x or be a vector of the last dim"
         bias_is_vector = int(bias.numel() == D and rows != 1)
     dev = _lib.require_device(*peers.tensors, x, bias, w, y)
-    stage_input(peers, x, rank)
+    peers = stage_input(peers, x, rank, stage)
     rc = peers.reduce_rmsnorm(rows, D, _lib.ptr(bias), bias_is_vector, w.data_ptr(), float(eps), y.data_ptr(),
                               _lib.current_stream(dev))
     _lib.check(rc, name)
@@ -49,6 +49,7 @@ def one_shot_all_reduce_bias_rms_norm(
     group=None,
     *,
     rank: int = 0,
+    stage: bool = False,
 ) -> None:
     """``y = rms_norm(bias + sum over the W slices, w, eps)``, one pass over the input.
 
@@ -58,9 +59,10 @@ def one_shot_all_reduce_bias_rms_norm(
     ``y = bf16(s * rsqrt(mean(s^2) + eps) * fp32(w))``.
 
     ``symm_mem_input`` is the ``[W, ...]`` stack or a list of W separate
-    tensors; ``x``, if given, is copied
-    into slice ``rank`` first (the reference's copy-in ``:57-61``), pass
-    ``None`` when the stack is already staged.  ``bias`` has the shape of
+    tensors; ``x``, if given, is read in place as rank ``rank``'s
+    contribution (the reference's copy-in ``:57-61`` serves the peers, of which there are none
+    here; ``stage=True`` also copies it into slice ``rank`` first); pass ``None`` when the stack
+    is already staged.  ``bias`` has the shape of
     ``x`` (reference usage) or ``[D]``.  ``BLOCK_SIZE``/``group`` are ignored.
     """
-    _launch_reduce_rms_norm("one_shot_all_reduce_bias_rms_norm", symm_mem_input, x, bias, w, y, eps, rank)
+    _launch_reduce_rms_norm("one_shot_all_reduce_bias_rms_norm", symm_mem_input, x, bias, w, y, eps, rank, stage)

@@ -17,6 +17,7 @@ def two_shot_all_reduce_bias(
     group=None,
     *,
     rank: int = 0,
+    stage: bool = False,
     layout: str = "rows",
     numel: int | None = None,
 ) -> torch.Tensor:
@@ -35,8 +36,8 @@ def two_shot_all_reduce_bias(
 
     ``symm_mem_input`` is the ``[W, ...]`` stack or a list of W separate
     tensors.  The message length is ``input_tensor.numel()`` if an input is given
-    (it is first copied into slice ``rank``, the reference's copy-in
-    ``:43-50``), else ``numel`` if passed, else ``bias.numel()`` for a
+    (it is read in place as rank ``rank``'s contribution; ``stage=True`` also
+    copies it into slice ``rank`` first, the reference's copy-in ``:43-50``), else ``numel`` if passed, else ``bias.numel()`` for a
     full-shape bias, else the slice size.  Returns ``output``.
     """
     peers = check_stack(symm_mem_input)
@@ -61,7 +62,7 @@ def two_shot_all_reduce_bias(
     if bias is not None:
         assert bias.dtype == torch.bfloat16 and bias.is_contiguous()
     dev = _lib.require_device(*peers.tensors, input_tensor, bias, output)
-    stage_input(peers, input_tensor, rank)
+    peers = stage_input(peers, input_tensor, rank, stage)
     lib = _lib.load()
     stream = _lib.current_stream(dev)
 

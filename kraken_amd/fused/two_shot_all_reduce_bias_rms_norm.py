@@ -19,6 +19,7 @@ def two_shot_all_reduce_bias_rms_norm(
     group=None,
     *,
     rank: int = 0,
+    stage: bool = False,
 ) -> None:
     """Same result as the one-shot variant; keeps the two-shot variant's shape rules.
 
@@ -46,4 +47,4 @@ def two_shot_all_reduce_bias_rms_norm(
     size_per_rank = rows_per_block * D // W
     assert size_per_rank * W == rows_per_block * D
     assert size_per_rank % 16 == 0
-    _launch_reduce_rms_norm("two_shot_all_reduce_bias_rms_norm", symm_mem_input, x, bias, w, y, eps, rank)
+    _launch_reduce_rms_norm("two_shot_all_reduce_bias_rms_norm", symm_mem_input, x, bias, w, y, eps, rank, stage)

@@ -287,3 +287,61 @@ def test_benchmark_helpers(dev):
     assert 0.5 < t_prof < 500
     assert benchmark_with_profiler(fn, r"no such kernel", warmup_iters=1, benchmark_iters=2) == 0.0
 
+
+
+def _device_kernels(fn):
+    """Names of the device kernels (and device copies) one call of fn enqueues."""
+    from torch.profiler import ProfilerActivity, profile
+
+    fn()
+    torch.cuda.synchronize()
+    with profile(activities=[ProfilerActivity.CUDA]) as prof:
+        fn()
+        torch.cuda.synchronize()
+    return [e.name for e in prof.events() if e.device_type == torch.autograd.DeviceType.CUDA]
+
+
+def test_input_is_read_in_place_by_one_kernel(dev):
+    """The reference stages this rank's input into its symmetric buffer inside the kernel
+    (kraken/fused/one_shot_all_reduce_bias.py:56-65).  Here the input is the rank's source where
+    it lies: one launch, no copy, the staged form's bits; stage=True keeps the side effect."""
+    W, rows, D, rank = 8, 16, 5120, 3
+    stack = orc.make_stack(W, (rows, D), seed0=5)
+    x = orc.randn_bf16((rows, D), 77)
+    bias, w = orc.randn_bf16((rows, D), 9), orc.randn_bf16((D,), 4, 0.02, 1.0)
+    staged = stack.clone()
+    staged[rank] = x
+    buf = torch.zeros(W, 1024, 1024, dtype=BF16, device=dev)          # larger than the message, as in the reference's tests
+    for r in range(W):
+        buf[r].view(-1)[: rows * D].copy_(stack[r].view(-1))
+    before = buf.clone()
+    xd, bd, wd = x.to(dev), bias.to(dev), w.to(dev)
+    out = torch.empty(rows, D, dtype=BF16, device=dev)
+    y = torch.empty(rows, D, dtype=BF16, device=dev)
+    calls = {
+        "one_shot_bias": lambda **kw: fused.one_shot_all_reduce_bias(buf, xd, bd, out, rank=rank, **kw),
+        "two_shot_bias": lambda **kw: fused.two_shot_all_reduce_bias(buf, xd, bd, out, rank=rank, **kw),
+        "one_shot_rms": lambda **kw: fused.one_shot_all_reduce_bias_rms_norm(buf, xd, bd, wd, y, rank=rank, **kw),
+        "two_shot_rms": lambda **kw: fused.two_shot_all_reduce_bias_rms_norm(buf, xd, bd, wd, y, rank=rank, **kw),
+    }
+    wants = {
+        "one_shot_bias": orc.reduce(staged, bias, bias_first=True),
+        "two_shot_bias": orc.reduce(staged, bias, bias_first=False),
+    }
+    for name, call in calls.items():
+        res = y if name.endswith("rms") else out
+        res.zero_()
+        kernels = _device_kernels(call)
+        assert len(kernels) == 1, kernels                              # no copy kernel, no memcpy
+        assert torch.equal(buf, before)                                # the buffer is left alone
+        in_place = res.clone()
+        if name in wants:
+            assert same_bits(in_place, wants[name])
+        else:
+            torch.testing.assert_close(in_place.cpu(), orc.reduce_bias_rms_norm(staged, bias, w), rtol=2e-2, atol=2e-2)
+        res.zero_()
+        kernels = _device_kernels(lambda: call(stage=True))
+        assert len(kernels) == 2, kernels                              # the copy-in, then the kernel
+        assert torch.equal(res, in_place)                              # the same bits
+        assert torch.equal(buf[rank].view(-1)[: rows * D], xd.view(-1))
+        buf.copy_(before)
