@@ -120,6 +120,8 @@ struct StackedPeers {
 // The KRAKEN_AMD_* environment variables (testing and tuning), read once per process and not on
 // every launch; kr_reload_env() reads them again.  -1 = not set.
 struct EnvSwitches {
+    int reduce_unroll;   // KRAKEN_AMD_REDUCE_UNROLL=1|2|4
+    int reduce_blocks;   // KRAKEN_AMD_REDUCE_BLOCKS=<n>
     int row_vpt;         // KRAKEN_AMD_ROW_VPT=1|2|4|8
     int row_lat;         // KRAKEN_AMD_ROW_LAT=0|1
     int row_split;       // KRAKEN_AMD_ROW_SPLIT=0|1

@@ -373,7 +373,7 @@ __global__ __launch_bounds__(256) void splitk_finish_kernel(const GemmArgs g, co
         return;
     }
     const int64_t off = (int64_t)mb * g.N + n;
-    if (!g.out_is_fp32 && g.n_peers > 0) unpack8(pack8(f), f);
+    if (!g.out_is_fp32) unpack8(pack8(f), f);   // the one-pass kernel rounds the product on its way to the epilogue
     for (int q = 0; q < g.n_peers; ++q) add8(ld_stream((const u32x4*)((const uint16_t*)g.peer.p[q] + off)), f);
     if (g.bias != nullptr) add8(*(const u32x4*)(g.bias + n), f);
     if (g.out_is_fp32) {

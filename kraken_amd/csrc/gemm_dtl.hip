@@ -695,14 +695,31 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_dtl_tail_finish_kernel(const
         return;
     }
     const int64_t off = (int64_t)mb * g.N + n;
-    for (int pq = 0; pq < g.n_peers; ++pq) {
-        const u32x2 w = *(const u32x2*)((const uint16_t*)g.peer.p[pq] + off);
-        sum.x += bf16_lo(w.x); sum.y += bf16_hi(w.x); sum.z += bf16_lo(w.y); sum.w += bf16_hi(w.y);
-    }
-    if (g.bias != nullptr) {
+    // The rounding of the main launch's tiles (gemm_dtl_tile): a tile that lies wholly in the band
+    // and adds its peers on the matrix cores (or has none) sums product, peers and bias in fp32 and
+    // rounds once; every other tile of a bf16 result rounds the product to bf16 first and adds the
+    // peers and the bias to that.
+    const bool tile_in_band = tile_m * BM >= g.band_row0 && tile_m * BM + BM <= g.band_row0 + g.band_rows;
+    const bool peers_exact = !g.mi16 && g.peers_on_mfma && g.n_peers > 0 && tile_in_band;
+    const bool bias_exact = g.bias != nullptr && tile_in_band && (g.n_peers == 0 || peers_exact);
+    auto add_peers = [&]() {
+        for (int pq = 0; pq < g.n_peers; ++pq) {
+            const u32x2 w = *(const u32x2*)((const uint16_t*)g.peer.p[pq] + off);
+            sum.x += bf16_lo(w.x); sum.y += bf16_hi(w.x); sum.z += bf16_lo(w.y); sum.w += bf16_hi(w.y);
+        }
+    };
+    auto add_bias = [&]() {
         const u32x2 w = *(const u32x2*)(g.bias + n);
         sum.x += bf16_lo(w.x); sum.y += bf16_hi(w.x); sum.z += bf16_lo(w.y); sum.w += bf16_hi(w.y);
+    };
+    if (peers_exact) add_peers();
+    if (bias_exact) add_bias();
+    if (!g.out_is_fp32) {
+        const uint32_t lo = pack_bf16(sum.x, sum.y), hi = pack_bf16(sum.z, sum.w);
+        sum = f32x4{bf16_lo(lo), bf16_hi(lo), bf16_lo(hi), bf16_hi(hi)};
     }
+    if (!peers_exact) add_peers();
+    if (g.bias != nullptr && !bias_exact) add_bias();
     if (g.out_is_fp32) *(f32x4*)((float*)g.out + off) = sum;
     else *(u32x2*)((uint16_t*)g.out + off) = u32x2{pack_bf16(sum.x, sum.y), pack_bf16(sum.z, sum.w)};
 }

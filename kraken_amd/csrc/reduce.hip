@@ -155,6 +155,7 @@ __global__ __launch_bounds__(kThreads) void reduce_rotated_kernel(
 // larger block wins whenever the blocks fill whole rounds of 256 CUs (32 MiB input: 9.0 -> 7.9 us,
 // 64 MiB: 16.0 -> 13.5 us), and loses 5 % at one and a half rounds.
 static int pick_unroll(int64_t nvec) {
+    if (const int u = env_switches().reduce_unroll; u == 1 || u == 2 || u == 4) return u;
     const int64_t blocks4 = (nvec + kThreads * 4 - 1) / (kThreads * 4);
     return (blocks4 >= 768 || (blocks4 >= 256 && blocks4 % 256 == 0)) ? 4 : 1;
 }
@@ -165,9 +166,13 @@ static void launch_reduce3(hipStream_t s, const SRC& tab, int W, int64_t nvec, c
     const int unroll = pick_unroll(nvec);
     const int64_t per_block = (int64_t)kThreads * unroll;
     int64_t blocks = (nvec + per_block - 1) / per_block;
-    if (blocks > kMaxBlocks) blocks = kMaxBlocks;
+    const int64_t max_blocks = env_switches().reduce_blocks > 0 ? env_switches().reduce_blocks : kMaxBlocks;
+    if (blocks > max_blocks) blocks = max_blocks;
     const dim3 grid((unsigned)blocks);
-    if (unroll == 4)
+    if (unroll == 2)
+        hipLaunchKernelGGL((reduce_kernel<SRC, WT, BIAS, BF, 2>), grid, dim3(kThreads), 0, s, tab, W, nvec, bias,
+                           d_vec, out);
+    else if (unroll == 4)
         hipLaunchKernelGGL((reduce_kernel<SRC, WT, BIAS, BF, 4>), grid, dim3(kThreads), 0, s, tab, W, nvec, bias,
                            d_vec, out);
     else

@@ -7,6 +7,8 @@ namespace kr {
 static EnvSwitches read_env() {
     EnvSwitches e;
     auto num = [](const char* name) { const char* t = getenv(name); return t != nullptr && t[0] != 0 ? atoi(t) : -1; };
+    e.reduce_unroll = num("KRAKEN_AMD_REDUCE_UNROLL");
+    e.reduce_blocks = num("KRAKEN_AMD_REDUCE_BLOCKS");
     e.row_vpt = num("KRAKEN_AMD_ROW_VPT");
     e.row_lat = num("KRAKEN_AMD_ROW_LAT");
     e.row_split = num("KRAKEN_AMD_ROW_SPLIT");

@@ -768,3 +768,38 @@ def test_gemm_paths_replay_from_a_graph(dev, monkeypatch):
         torch.cuda.synchronize()
         for e, r in zip(eager, got):
             assert torch.equal(e, r)
+
+
+@pytest.mark.parametrize("peers_mode", ["epilogue", "mfma"])
+@pytest.mark.parametrize("mfma", ["16", "32"])
+def test_split_tiles_round_like_unsplit_tiles(dev, monkeypatch, peers_mode, mfma):
+    """Tiles whose K loop is split (tail round, finished by a separate pass) and tiles of the main
+    launch must round alike: with small-integer operands and peers and bias on a grid of 1/16
+    every fp32 sum is exact whatever its order, so the split result has to equal the unsplit one
+    bit for bit -- with peers and bias on a bf16 result, where rounding the product before or after
+    the peers are added makes a visible difference."""
+    M, N, K, P = 4352, 4096, 1024, 3          # 272 tiles of 256 x 256: 256 + 16 in the tail
+    g = torch.Generator().manual_seed(5)
+    a = torch.randint(-3, 4, (M, K), generator=g).to(BF16)
+    b = torch.randint(-3, 4, (K, N), generator=g).to(BF16)
+    peers = (torch.randint(-127, 128, (P, M, N), generator=g).float() / 16).to(BF16)
+    bias = (torch.randint(-32, 33, (N,), generator=g).float() / 4).to(BF16)
+    ad, bd, pd, biasd = a.to(dev), b.to(dev), peers.to(dev), bias.to(dev)
+    monkeypatch.setenv("KRAKEN_AMD_GEMM_PEERS", peers_mode)
+    monkeypatch.setenv("KRAKEN_AMD_GEMM_MFMA", mfma)
+    res = {}
+    for split in ("0", "3"):
+        monkeypatch.setenv("KRAKEN_AMD_GEMM_TAILSPLIT", split)
+        res[split] = [
+            fused.gemm_one_shot_all_reduce_fused(ad, bd, peers=pd, bias=biasd, out_dtype=BF16),
+            fused.gemm_one_shot_all_reduce_fused(ad, bd, bias=biasd, out_dtype=BF16),
+            fused.gemm_one_shot_all_reduce_fused(ad, bd, peers=pd, bias=biasd),
+            fused.gemm_reduce_scatter(ad, bd, peers=pd[:1, : M // 2].contiguous(), rank=1, world_size=2),
+        ]
+    for x, y in zip(res["0"], res["3"]):
+        assert torch.equal(x, y)
+    # the exact product is large enough for the two rounding orders to differ somewhere
+    prod = a.float() @ b.float()
+    once = (prod + peers.float().sum(0) + bias.float()).to(BF16)
+    twice = (prod.to(BF16).float() + peers.float().sum(0) + bias.float()).to(BF16)
+    assert not torch.equal(once, twice)
