@@ -19,6 +19,9 @@ __global__ __launch_bounds__(kWave) void write_value32_kernel(uint32_t* addr, ui
 __global__ __launch_bounds__(kWave) void wait_value32_kernel(const uint32_t* addr, uint32_t value, uint64_t ticks,
                                                              int* status) {
     if (threadIdx.x != 0) return;
+    // a wait earlier on this stream that shares the status word has already run out: the flags are
+    // not coming, and waiting for each of them in turn would only add the limit once per wait
+    if (status != nullptr && __hip_atomic_load(status, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM) != 0) return;
     const uint64_t t0 = __builtin_amdgcn_s_memrealtime();
     while (__hip_atomic_load(addr, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM) != value) {
         if (__builtin_amdgcn_s_memrealtime() - t0 > ticks) {

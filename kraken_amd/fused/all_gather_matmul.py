@@ -3,7 +3,7 @@ from __future__ import annotations
 
 import torch
 
-from .. import _lib
+from .. import _lib, _waits
 from ..comm._common import PeerBuffers
 from ..comm.copy_engine_all_gather import _copy_engine_all_gather_w_progress
 from . import _gemm
@@ -64,7 +64,10 @@ def all_gather_matmul(
       (``rank``) read it in place, every other tile waits for its chunk's flag
       (``:95-110``).  The current stream then waits for the side stream
       (``:316``).  ``status`` (int32 ``[1]``, zeroed by the caller) receives a
-      non-zero value if a tile's wait ran out (``wait_limit_us``, default 5 s).
+      non-zero value if a tile's wait ran out (``wait_limit_us``, default 5 s) and
+      ``c`` is then invalid; without ``status`` the wrapper keeps a word of its own
+      and the next call of an overlap function (or ``kraken_amd._waits.check()``)
+      raises once the failed call has finished.
       The copies are ordinary copy kernels, which share the compute units with
       the GEMM; ``copy_engine=True`` hands them to the GPU's copy engines.
 
@@ -120,6 +123,13 @@ def all_gather_matmul(
                                                         copy_engine=kwargs.get("copy_engine", False))
     configs = {"RANK": rank, "WORLD_SIZE": W, "SPLITS_PER_RANK": splits,
                "wait_limit_us": kwargs.get("wait_limit_us", 0)}
-    c = _matmul_w_progress(a_out, peers.slice(rank), b, progress, configs, kwargs.get("status"))
+    _waits.check()
+    status = kwargs.get("status")
+    own_status = status is None
+    if own_status:
+        status = _waits.new_status(dev)
+    c = _matmul_w_progress(a_out, peers.slice(rank), b, progress, configs, status)
     torch.cuda.current_stream(dev).wait_stream(backend_stream)
+    if own_status:
+        _waits.watch(status, "all_gather_matmul")
     return a_out, c

@@ -3,7 +3,7 @@ from __future__ import annotations
 
 import torch
 
-from .. import _lib
+from .. import _lib, _waits
 from ..comm.copy_engine_all_gather import _get_backend_stream
 from . import _gemm
 
@@ -96,7 +96,9 @@ def copy_engine_scatter(
     a sequence of W tensors ``[M/W, N]`` (``None`` entries are skipped: no wait, no
     copy); ``output[r]`` stands for slot ``rank`` of rank r's symmetric buffer
     (``:165-169``).  The waits are bounded (``wait_limit_us``, default 5 s); a wait
-    that runs out sets ``status`` (int32 ``[1]``, zeroed by the caller) to 1.  The
+    that runs out sets ``status`` (int32 ``[1]``, zeroed by the caller) to 1 and the bands copied
+    behind it are invalid; without ``status`` the wrapper keeps a word of its own and the next call
+    of an overlap function (or ``kraken_amd._waits.check()``) raises once the copies have run.  The
     copies are ordinary copy kernels; ``copy_engine=True`` hands them to the GPU's
     copy engines (``kr_copy_engine_memcpy``).
     """
@@ -108,6 +110,10 @@ def copy_engine_scatter(
     dev = _lib.require_device(inp, signal_pad, status, *[t for t in output if t is not None])
     lib = _lib.load()
     stream = _lib.current_stream(dev)
+    _waits.check()
+    own_status = status is None
+    if own_status:
+        status = _waits.new_status(dev)     # shared by the W waits: after one runs out the others give up at once
     for step in range(W):
         remote = (rank + step + 1) % W
         dst = output[remote]
@@ -121,6 +127,8 @@ def copy_engine_scatter(
             _lib.copy_engine_copy(dst, band, stream)
         else:
             dst.copy_(band)
+    if own_status:
+        _waits.watch(status, "copy_engine_scatter")
 
 
 def gemm_reduce_scatter_ce_persistent(

@@ -413,6 +413,40 @@ def test_copy_engine_scatter_wait_is_bounded(dev):
     assert ok.item() == 0 and torch.equal(outs[0], inp[:rows])
 
 
+def test_bounded_waits_without_a_status_do_not_fail_silently(dev):
+    """No `status` passed: the wrappers keep a word of their own, every wait of the call shares it
+    (after the first one runs out the others give up at once), and the failure is raised on the
+    next look -- here by an explicit check, in use by the next call of an overlap function."""
+    import time
+    from kraken_amd import _waits
+    from kraken_amd._lib import KrakenAmdError
+    from kraken_amd.fused.gemm_reduce_scatter_ce_persistent import copy_engine_scatter
+    W, rows, N = 8, 64, 128
+    inp = torch.ones(W * rows, N, dtype=BF16, device=dev)
+    outs = [torch.zeros(rows, N, dtype=BF16, device=dev) for _ in range(W)]
+    _waits.check(block=True)                                              # nothing pending from earlier tests
+    copy_engine_scatter(inp, outs, torch.ones(W, dtype=torch.int32, device=dev), rank=0)      # every flag is set
+    _waits.check(block=True)
+    never = torch.zeros(W, dtype=torch.int32, device=dev)                 # no flag ever comes: 8 waits of 20 ms
+    t0 = time.perf_counter()
+    copy_engine_scatter(inp, outs, never, rank=0, wait_limit_us=20000)
+    with pytest.raises(KrakenAmdError, match="copy_engine_scatter.*ran out"):
+        _waits.check(block=True)
+    assert time.perf_counter() - t0 < 0.1                                 # one limit, not eight
+    _waits.check(block=True)                                              # reported once
+    # the all-gather matmul with chunks that never arrive (no copies are enqueued for this call)
+    from kraken_amd.fused.all_gather_matmul import _matmul_w_progress
+    m, K, Nn = 64, 128, 256
+    a = orc.randn_bf16((4 * m, K), 1).to(dev)
+    bT = orc.randn_bf16((Nn, K), 2, 0.05).to(dev)
+    status = _waits.new_status(dev)
+    _matmul_w_progress(a, a[:m], bT.T, torch.zeros(4, dtype=torch.int32, device=dev),
+                       {"RANK": 0, "WORLD_SIZE": 4, "SPLITS_PER_RANK": 1, "wait_limit_us": 2000}, status)
+    _waits.watch(status, "all_gather_matmul")
+    with pytest.raises(KrakenAmdError, match="all_gather_matmul"):
+        _waits.check(block=True)
+
+
 def test_ce_persistent_reference_shape(dev):
     """(8192, 4096, 14336), the shape of test/test_gemm_reduce_scatter.py:93-111 (tolerance 1e-2
     there; the gate here is the library's 2e-2 on sampled rows)."""
