@@ -176,8 +176,11 @@ int kr_rmsnorm_bf16(const void* x, const void* w, float eps, int64_t rows, int64
  * of 256x256, K % 64 == 0) and a band of at least half the rows, the peers of
  * tiles lying wholly in the band are added on the matrix cores, where an
  * Inf/NaN in a peer also turns the rest of the aligned 32-column block of its
- * row into NaN; KRAKEN_AMD_GEMM_PEERS=epilogue in the environment keeps such
- * values in their own element (as calls with a smaller band always do).
+ * row into NaN.  This default DEVIATES from the reference, whose epilogue adds the
+ * peers element by element (gemm_one_shot_all_reduce_fused.py:85-92) and so keeps a
+ * non-finite value in its own element; finite inputs give the same results either
+ * way.  KRAKEN_AMD_GEMM_PEERS=epilogue in the environment selects the reference's
+ * behaviour (as calls with a smaller band, and the 16x16x32 form, always have).
  *
  * Replaces
  *   kraken/fused/gemm_one_shot_all_reduce_fused.py:56-99   (band = all rows)
