@@ -28,6 +28,10 @@ HIPCC_FLAGS = [
     "-fPIC",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-Wno-unused-command-line-argument",
+    "-Wno-inline-asm",
+    # the k-steps of the GEMM kernels are fully unrolled by "#pragma unroll"; above the default limit
+    # (16384 instructions) the request is dropped without a word and register arrays turn into scratch
+    "-mllvm", "-pragma-unroll-threshold=1048576",
 ]
 
 
