@@ -43,7 +43,16 @@ W = 8
 # hardware counters itself; the figures and the commands behind them are kept as text under
 # profiles/ (one file per kernel and workload).  None: not measured.
 MEASURED_TRAFFIC = {
-    "one_shot_reduce_w8_4096x4096": 302054820,
+    "one_shot_reduce_w8_4096x4096": 302053204,              # profiles/reduce_kernel_w8_4096x4096.md
+    "two_shot_share_w8_512x4096": 37839283,                 # profiles/reduce_kernel_w8_two_shot_share_512x4096.md
+    "reduce_bias_rmsnorm_w8_256x4096": 19050022,            # profiles/reduce_rmsnorm_kernel_w8_256x4096.md
+    "reduce_bias_rmsnorm_w8_16x8192_decode": 2483922,       # profiles/reduce_rmsnorm_split_kernel_w8_16x8192.md
+    "reduce_bias_rmsnorm_w8_16384x4096_large": 1208025963,  # profiles/reduce_rmsnorm_kernel_w8_16384x4096.md
+    # the GEMMs: L2 fills (A and B panels re-read per tile row / column, served mostly by the 256 MB
+    # last-level cache, not by HBM) + write-backs
+    "gemm_reduce_scatter_8192x8192x3584_w8": 962243626,     # profiles/gemm_dtl16_kernel_reduce_scatter_8192x8192x3584.md
+    "gemm_all_reduce_4096x8192x1024_w8": 705354977,         # profiles/gemm_dtl_kernel_all_reduce_4096x8192x1024.md
+    "all_gather_matmul_8192x3584x8192_w8": 875039914,       # profiles/gemm_dtl16_kernel_all_gather_matmul_8192x3584x8192.md
 }
 
 # Targets of the benchmark definition: fraction of the binding roof.  The W = 8 reduce(+bias+RMSNorm)
@@ -222,7 +231,11 @@ class ReduceBiasRmsNorm(Workload):
         return orc.reduce_bias_rms_norm_library(self.host, self.hbias, self.hw, 1e-5)
 
     def describe(self):
-        return {"W": W, "shape": [W, self.rows, self.D], "eps": 1e-5, "kernel": "reduce_rmsnorm_kernel"}
+        from kraken_amd import _lib
+
+        split = _lib.load().kr_rmsnorm_workspace_bytes(W, self.rows, self.D) > 0
+        return {"W": W, "shape": [W, self.rows, self.D], "eps": 1e-5,
+                "kernel": "reduce_rmsnorm_split_kernel" if split else "reduce_rmsnorm_kernel"}
 
 
 class GemmReduceScatter(Workload):
