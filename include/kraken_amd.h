@@ -12,7 +12,9 @@
  *   - all data pointers are DEVICE pointers; bf16 = 2-byte bfloat16;
  *   - `stream` is a hipStream_t (NULL = the default stream); a call enqueues
  *     its kernel(s) on that stream and returns without synchronising;
- *   - the library keeps no state between calls and is re-entrant;
+ *   - the library keeps no state between calls and is re-entrant (two exceptions, both named
+ *     where they apply: the tuning switches of the environment are read once per process, and
+ *     kr_gemm_reduce_noalloc_bf16 uses a device array of the library's own);
  *   - return value: 0 on success; a negative KR_ERR_* code when the arguments
  *     are rejected on the host BEFORE anything is launched (so argument
  *     validation can be exercised on a machine without a GPU); a positive
