@@ -48,9 +48,12 @@ def gemm_producer_w_progress(
     finished tile is counted into ``progress[r]`` of the bands it touches and the
     tile that completes band ``r`` sets ``signal_pad[r] = 1`` (``:117-132``).  Both
     are 32-bit integer tensors of ``WORLD_SIZE`` elements, zeroed by the caller
-    (``:364-365``).  Shapes with so few output tiles that the library splits their
-    K loop over several workgroups finish all bands together: their flags are set
-    by a stream-ordered fill behind the GEMM and ``progress`` is not counted.
+    (``:364-365``).  Shapes whose output tiles all run at once (one round of the
+    compute units or less) finish all bands together, so for those the library's
+    fastest GEMM is used when it is a split one (K loop shared between workgroups):
+    their flags are set by a stream-ordered fill behind the GEMM and ``progress``
+    is not counted.  Every larger shape runs the producer kernel, whose bands
+    finish, and are flagged, one after the other.
     """
     a2, b2 = _gemm.prepare_operands(a, b)
     M, N = a2.shape[0], b2.shape[1]
@@ -62,7 +65,8 @@ def gemm_producer_w_progress(
     dev = _lib.require_device(a2, b2, gemm_out, progress, signal_pad)
     lib = _lib.load()
     pivot = ((rank + 1) % W) * (M // W)
-    if lib.kr_gemm_workspace_bytes(M, N, a2.shape[1]) > 0:
+    one_round = -(-M // 256) * -(-N // 256) <= torch.cuda.get_device_properties(dev).multi_processor_count
+    if one_round and lib.kr_gemm_workspace_bytes(M, N, a2.shape[1]) > 0:
         _gemm.launch("gemm_producer_w_progress", a2, b2, M, N, None, 0, 0, None, 0, 0, gemm_out, None, pivot)
         signal_pad.fill_(1)
         return

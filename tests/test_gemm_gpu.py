@@ -318,6 +318,27 @@ def test_producer_gemm_flags_every_band(dev, tile, shape, W, rank):
     torch.testing.assert_close(gemm_out.cpu(), (a.float() @ b.float()).to(BF16), **TOL)
 
 
+def test_producer_gemm_counts_bands_of_a_shape_with_a_partial_last_round(dev):
+    """272 tiles of 256 x 256 = one round of the compute units and a partial second one: the plain GEMM
+    would split that tail over idle compute units (a workspace is asked for), the producer keeps the
+    one-pass kernel so that every band is counted and flagged when it is finished."""
+    from kraken_amd import _lib
+    from kraken_amd.fused.gemm_reduce_scatter_ce_persistent import gemm_producer_w_progress
+    M, N, K, W, rank = 4352, 4096, 4096, 8, 3
+    assert _lib.load().kr_gemm_workspace_bytes(M, N, K) > 0
+    g = torch.Generator().manual_seed(11)
+    a = (torch.randn(M, K, generator=g) * 0.25).to(BF16)
+    b = (torch.randn(K, N, generator=g) * 0.25).to(BF16)
+    gemm_out = torch.full((M, N), float("nan"), dtype=BF16, device=dev)
+    progress = torch.zeros(W, dtype=torch.int32, device=dev)
+    signal_pad = torch.zeros(W, dtype=torch.int32, device=dev)
+    gemm_producer_w_progress(a.to(dev), b.to(dev), gemm_out, progress, signal_pad, {"RANK": rank, "WORLD_SIZE": W})
+    torch.cuda.synchronize()
+    assert signal_pad.tolist() == [1] * W
+    assert progress.tolist() == _band_tile_counts(M, N, W, 256)
+    torch.testing.assert_close(gemm_out.cpu(), (a.float() @ b.float()).to(BF16), **TOL)
+
+
 @pytest.mark.parametrize("rank", [0, 2])
 def test_copy_engine_scatter_overlaps_the_producer(dev, tile, rank):
     """The reference's overlap: the band copies sit on a side stream behind stream-ordered waits
