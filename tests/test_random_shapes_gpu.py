@@ -140,3 +140,48 @@ def test_all_gather_matmul_random_shapes(dev, seed):
     a_got, c_got = fused.all_gather_matmul(stack.to(dev), bT.to(dev).T, rank=rank)
     assert same_bits(a_got, a_want)
     torch.testing.assert_close(c_got.cpu(), c_want, **TOL)
+
+
+@pytest.mark.parametrize("seed", range(24))
+def test_large_tile_kernel_random_shapes_and_switches(dev, monkeypatch, seed):
+    """The 256 x 256 kernel forced on shapes it would not be chosen for, with a random draw of its
+    variants: 16x16x32 or 32x32x16 matrix-core blocks, peers added on the matrix cores or in the
+    epilogue, either layout of B, ragged edges, a reduce band that starts and ends inside tiles,
+    a forced split of the last tiles' K loops."""
+    rnd = random.Random(6000 + seed)
+    monkeypatch.setenv("KRAKEN_AMD_GEMM_TILE", "256")
+    monkeypatch.setenv("KRAKEN_AMD_GEMM_MFMA", rnd.choice(["16", "32"]))
+    monkeypatch.setenv("KRAKEN_AMD_GEMM_PEERS", rnd.choice(["mfma", "epilogue"]))
+    if rnd.random() < 0.3:
+        monkeypatch.setenv("KRAKEN_AMD_GEMM_TAILSPLIT", rnd.choice(["2", "3"]))
+    W = rnd.choice([1, 2, 4, 8])
+    M = W * rnd.choice([32, 64, 65, 128, 160, 256])
+    N = 8 * rnd.choice([32, 33, 64, 65, 96, 128])
+    K = 64 * rnd.choice([1, 2, 3, 4, 8, 16])
+    rank = rnd.randrange(W)
+    b_t = rnd.random() < 0.5
+    a = orc.randn_bf16((M, K), 72 + seed)
+    b = orc.randn_bf16((N, K), 73 + seed, 0.05).T if b_t else orc.randn_bf16((K, N), 73 + seed, 0.05)
+    ad, bd = a.to(dev), b.to(dev)
+    if rnd.random() < 0.5:
+        peers = torch.stack([orc.randn_bf16((M // W, N), 300 + j + seed) for j in range(W - 1)]) if W > 1 else None
+        want, c_want = orc.gemm_reduce_scatter(a, b, peers, rank, W)
+        c_scratch = torch.full((M, N), float("nan"), dtype=BF16, device=dev)
+        out = fused.gemm_reduce_scatter(ad, bd, peers=None if peers is None else peers.to(dev), rank=rank,
+                                        c_scratch=c_scratch, world_size=W)
+        torch.testing.assert_close(out.cpu(), want, **TOL)
+        other = torch.ones(M, dtype=torch.bool)
+        other[rank * (M // W):(rank + 1) * (M // W)] = False
+        torch.testing.assert_close(c_scratch.cpu()[other], c_want[other], **TOL)
+        assert torch.isnan(c_scratch.cpu()[~other].float()).all()
+    else:
+        P = rnd.choice([0, 1, 7])
+        peers = torch.stack([orc.randn_bf16((M, N), 400 + j + seed) for j in range(P)]) if P else None
+        bias = orc.randn_bf16((N,), 9 + seed, 0.02) if rnd.random() < 0.6 else None
+        pd = None if peers is None else peers.to(dev)
+        bsd = None if bias is None else bias.to(dev)
+        want = orc.gemm_all_reduce(a, b, peers, bias)
+        torch.testing.assert_close(fused.gemm_one_shot_all_reduce_fused(ad, bd, peers=pd, bias=bsd).cpu(), want,
+                                   rtol=1e-3, atol=1e-3)
+        torch.testing.assert_close(fused.gemm_one_shot_all_reduce_fused(ad, bd, peers=pd, bias=bsd, out_dtype=BF16).cpu(),
+                                   want.to(BF16), **TOL)
