@@ -133,6 +133,10 @@ int kr_reduce_rmsnorm_bf16(const void* stack, int W, int64_t slice_stride, int64
  * captured graph; clearing it again between calls is harmless).  Calls that use one workspace
  * must not overlap (same stream, or otherwise ordered).  workspace == NULL, a workspace that is
  * too small, or a shape that does not profit: exactly the entry point without workspace.
+ * The exchange is a bounded wait (seconds; the wavefronts of a row run at the same time, so it
+ * normally lasts a microsecond): a row whose wavefronts did not meet within the bound, which only
+ * a workspace shared by overlapping calls or a GPU that other work keeps full for that long can
+ * cause, is written as NaN.
  * No counterpart in the reference (one 1024-thread CTA per row whatever the shape,
  * kraken/fused/one_shot_all_reduce_bias_rms_norm.py:144-145).
  */

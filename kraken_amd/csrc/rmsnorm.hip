@@ -171,7 +171,9 @@ __global__ __launch_bounds__(kMaxThreads) void reduce_rmsnorm_kernel(
 // agent scope (they are served by the memory side, about 1 us a round trip, which is the price
 // of the exchange).  All wavefronts of a row are resident together (the grid is at most
 // kSplitMaxWaves one-wave workgroups, dispatched in order), so the poll ends; it is bounded all
-// the same and falls through after kSplitSpinLimit polls.
+// the same: after kSplitSpinLimit polls (seconds) the wavefront gives up and its piece of the row
+// is written as NaN.  Tags are 32 bits: a slot left by an earlier call could only be mistaken for
+// a fresh one if exactly 2^32 calls on the workspace lay between two uses of that slot.
 constexpr int kSplitSlots = 64;                       // wavefronts per row at most -> D <= 32768
 constexpr int kSplitMaxRows = 64;
 constexpr int kSplitMaxWaves = 1024;
@@ -219,17 +221,19 @@ __global__ __launch_bounds__(kWave) void reduce_rmsnorm_split_kernel(
         __hip_atomic_store(slots + piece, ((uint64_t)tag << 32) | __builtin_bit_cast(uint32_t, ss), __ATOMIC_RELAXED,
                            __HIP_MEMORY_SCOPE_AGENT);
     uint64_t v = (uint64_t)tag << 32;
-    for (int spin = 0; spin < kSplitSpinLimit; ++spin) {
+    bool met = false;
+    for (int spin = 0; spin < kSplitSpinLimit && !met; ++spin) {
         if (lane < nw) v = __hip_atomic_load(slots + lane, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        if (__all((uint32_t)(v >> 32) == tag)) break;
-        __builtin_amdgcn_s_sleep(1);
+        met = __all((uint32_t)(v >> 32) == tag);
+        if (!met) __builtin_amdgcn_s_sleep(1);
     }
     if (piece == 0 && lane == 0)
         __hip_atomic_store(block, (uint64_t)tag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     float total = 0.0f;
     const int part = (int)(uint32_t)v;
     for (int k = 0; k < nw; ++k) total += __builtin_bit_cast(float, __builtin_amdgcn_readlane(part, k));
-    const float rstd = __builtin_amdgcn_rsqf(total * inv_d + eps);
+    // a row whose wavefronts did not meet within the bound comes out as NaN, not as a plausible wrong value
+    const float rstd = met ? __builtin_amdgcn_rsqf(total * inv_d + eps) : __builtin_nanf("");
 
     if (c < d_vec) {
         float wf[8], o[8];
