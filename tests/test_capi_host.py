@@ -378,3 +378,14 @@ def test_missing_library_fails_loudly(monkeypatch, tmp_path):
     monkeypatch.setattr(_lib, "LIB_PATH", tmp_path / "libkraken_amd.so")
     with pytest.raises(RuntimeError, match="kraken_amd.build"):
         _lib.load()
+
+
+def test_bench_refuses_more_than_one_gpu():
+    """bench.py measures one rank on one GPU: any other --gpus value ends with a message and exit status 2
+    before anything touches a device."""
+    import subprocess
+    import sys
+    r = subprocess.run([sys.executable, str(Path(__file__).resolve().parents[1] / "bench.py"), "--gpus", "2"],
+                       capture_output=True, text=True, timeout=120)
+    assert r.returncode == 2
+    assert "--gpus 2 is not supported" in r.stderr and r.stdout == ""
