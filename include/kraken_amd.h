@@ -136,17 +136,25 @@ int kr_reduce_rmsnorm_bf16(const void* stack, int W, int64_t slice_stride, int64
  * The exchange is a bounded wait (seconds; the wavefronts of a row run at the same time, so it
  * normally lasts a microsecond): a row whose wavefronts did not meet within the bound, which only
  * a workspace shared by overlapping calls or a GPU that other work keeps full for that long can
- * cause, is written as NaN.
+ * cause, is written as NaN, and 1 + the row's index is stored to *status (device int32, 4-byte
+ * aligned, may be NULL; zeroed by the caller; never written otherwise).  After such a time-out the
+ * workspace must be zeroed again before its next use (a late wavefront of the failed call may
+ * have left a slot that the next call would take for a fresh one).  The wavefronts of a row can
+ * only meet if all of them are resident together: the launch is at most 1024 one-wave workgroups,
+ * which an otherwise idle GPU starts at once, but a kernel on another stream that keeps every
+ * compute unit full (a GEMM, say) can delay some of them by its own run time.
  * No counterpart in the reference (one 1024-thread CTA per row whatever the shape,
  * kraken/fused/one_shot_all_reduce_bias_rms_norm.py:144-145).
  */
 int64_t kr_rmsnorm_workspace_bytes(int W, int64_t rows, int64_t D);
 int kr_reduce_rmsnorm_ws_bf16(const void* stack, int W, int64_t slice_stride, int64_t rows, int64_t D,
                               const void* bias, int bias_is_vector, const void* w, float eps,
-                              void* y, void* workspace, int64_t workspace_bytes, void* stream);
+                              void* y, void* workspace, int64_t workspace_bytes, int32_t* status,
+                              void* stream);
 int kr_reduce_rmsnorm_ptrs_ws_bf16(const void* const* bufs, int W, int64_t rows, int64_t D,
                                    const void* bias, int bias_is_vector, const void* w, float eps,
-                                   void* y, void* workspace, int64_t workspace_bytes, void* stream);
+                                   void* y, void* workspace, int64_t workspace_bytes, int32_t* status,
+                                   void* stream);
 
 /*
  * Stand-alone RMSNorm: y = bf16( x * rsqrt(mean(x^2) + eps) * w ), row-wise.
@@ -299,8 +307,17 @@ int kr_gemm_reduce_ptrs_ws_bf16(const void* A, int64_t lda_m, int64_t lda_k,
  * ordering between them, or several host threads) race on it and must be serialised by the
  * caller.  Nothing in the array has to start at zero (the first launch overwrites every word
  * the second reads), so a call leaves nothing behind that a later call depends on.
+ * The first use on a device looks the array up (hipGetSymbolAddress), which can make the HIP
+ * runtime load the library's code for that device and with it allocate the array: call kr_init()
+ * once per device, with that device current and outside any graph capture, before the first call
+ * that must not allocate.  The array used is the one of the device that is current at the call,
+ * which must be the device `stream` belongs to (as for any launch).
  */
 #define KR_STATIC_SCRATCH_BYTES (64ll << 20)
+/* Loads the library's device code for the current device and resolves its scratch array, so that
+ * no later call has to (0, or the hipError_t of the lookup).  Idempotent and thread-safe; it has no
+ * counterpart in the reference and is needed only by callers of kr_gemm_reduce_noalloc_bf16. */
+int kr_init(void);
 int kr_gemm_reduce_noalloc_bf16(const void* A, int64_t lda_m, int64_t lda_k,
                                 const void* B, int64_t ldb_k, int64_t ldb_n,
                                 int64_t M, int64_t N, int64_t K,
@@ -425,6 +442,37 @@ int kr_copy_engine_memcpy(void* dst, const void* src, int64_t bytes, void* strea
  */
 int kr_reduce_rotated_bf16(const void* in, int W, int64_t rows, int64_t N, int rank,
                            int acc_bf16, void* out, void* stream);
+
+/*
+ * Which kernel kr_gemm_reduce_*_bf16 would run for a shape (contiguous operands), decided by the
+ * same code that launches it; for benchmarks and logs that want to name the kernel they timed.
+ * No counterpart in the reference (its tile sizes are keyword arguments of the wrappers,
+ * kraken/fused/gemm_one_shot_all_reduce_fused.py:128-133).  Nothing is launched.
+ *   b_transposed: B is given transposed-contiguous ([N, K] memory); 0: row-major [K, N]
+ *   workspace_bytes: size of the workspace the call would be given (0: none)
+ *   plan[0] workgroup tile: 256 (256x256 tile, global->LDS loads without registers) or 128
+ *   plan[1] matrix-core block of the k loop: 16 (v_mfma_f32_16x16x32_bf16) or 32 (32x32x16)
+ *   plan[2] 128 tile: workgroups per tile that share its K loop (1: one pass)
+ *   plan[3] 256 tile: tiles of the last partial round that are split, plan[4] parts of each
+ *   plan[5] column panels per scheduling group
+ *   plan[6] 1: tiles that lie wholly in the reduce band add the peers on the matrix cores
+ *   plan[7] 1: M or N is not a multiple of the tile (bounds-checked edge tiles)
+ */
+int kr_gemm_plan(int64_t M, int64_t N, int64_t K, int b_transposed, int n_peers, int64_t band_rows,
+                 int has_bias, int has_c_full, int64_t workspace_bytes, int32_t plan[8]);
+
+/*
+ * Measurement aids, without a counterpart in the reference: the plainest kernels that move a
+ * given number of bytes, so that a benchmark can state what a launch of that size costs on this
+ * machine before any arithmetic is added.
+ *   kr_probe_read: every byte of [src, src + bytes) is loaded once (128-bit non-temporal loads,
+ *     one per thread up to 16 MiB, 256-thread workgroups); nothing is written.  `sink` may be
+ *     NULL (it only keeps the loads alive for the compiler).
+ *   kr_probe_copy: the same loads, each followed by a 128-bit non-temporal store to dst.
+ * bytes % 16 == 0; src, dst 16-byte aligned; bytes == 0: nothing is launched.
+ */
+int kr_probe_read(const void* src, int64_t bytes, void* sink, void* stream);
+int kr_probe_copy(const void* src, void* dst, int64_t bytes, void* stream);
 
 #ifdef __cplusplus
 }

@@ -25,6 +25,7 @@ KR_ERR_SCRATCH = -11
 
 _SIGNATURES = {
     "kr_version": (c_int, []),
+    "kr_init": (c_int, []),
     "kr_strerror": (c_char_p, [c_int]),
     "kr_reload_env": (None, []),
     "kr_reduce_bf16": (
@@ -61,12 +62,12 @@ _SIGNATURES = {
     "kr_reduce_rmsnorm_ws_bf16": (
         c_int,
         [c_void_p, c_int, c_int64, c_int64, c_int64, c_void_p, c_int, c_void_p, c_float, c_void_p,
-         c_void_p, c_int64, c_void_p],
+         c_void_p, c_int64, c_void_p, c_void_p],
     ),
     "kr_reduce_rmsnorm_ptrs_ws_bf16": (
         c_int,
         [c_void_p, c_int, c_int64, c_int64, c_void_p, c_int, c_void_p, c_float, c_void_p,
-         c_void_p, c_int64, c_void_p],
+         c_void_p, c_int64, c_void_p, c_void_p],
     ),
     "kr_rmsnorm_bf16": (c_int, [c_void_p, c_void_p, c_float, c_int64, c_int64, c_void_p, c_void_p]),
     "kr_gemm_reduce_bf16": (
@@ -107,6 +108,9 @@ _SIGNATURES = {
     "kr_copy_engine_memcpy": (c_int, [c_void_p, c_void_p, c_int64, c_void_p]),
     "kr_flag_arrive_wait": (c_int, [c_void_p, c_int, c_int, c_int64, c_void_p, c_void_p]),
     "kr_reduce_rotated_bf16": (c_int, [c_void_p, c_int, c_int64, c_int64, c_int, c_int, c_void_p, c_void_p]),
+    "kr_gemm_plan": (c_int, [c_int64, c_int64, c_int64, c_int, c_int, c_int64, c_int, c_int, c_int64, c_void_p]),
+    "kr_probe_read": (c_int, [c_void_p, c_int64, c_void_p, c_void_p]),
+    "kr_probe_copy": (c_int, [c_void_p, c_void_p, c_int64, c_void_p]),
 }
 
 EXPORTS = tuple(_SIGNATURES)
@@ -134,6 +138,24 @@ def load() -> ctypes.CDLL:
             fn.argtypes = argtypes
         _lib = lib
     return _lib
+
+
+def gemm_plan(M: int, N: int, K: int, b_transposed: bool, n_peers: int = 0, band_rows: int | None = None,
+              has_bias: bool = False, has_c_full: bool = False, workspace_bytes: int = 0) -> dict:
+    """The kernel ``kr_gemm_reduce_*_bf16`` picks for a shape (``kr_gemm_plan``), as a dict with the
+    kernel's name as a profiler lists it."""
+    plan = (ctypes.c_int32 * 8)()
+    rc = load().kr_gemm_plan(M, N, K, int(b_transposed), n_peers, M if band_rows is None else band_rows,
+                             int(has_bias), int(has_c_full), workspace_bytes, plan)
+    check(rc, "gemm_plan")
+    tile, block, splits, tail, tail_splits, group_n, mfma_peers, ragged = list(plan)
+    if tile == 256:
+        kernel = "gemm_dtl16_kernel" if block == 16 else "gemm_dtl_kernel"
+    else:
+        kernel = "gemm_reduce_kernel"
+    return {"kernel": kernel, "tile": tile, "mfma": "16x16x32" if block == 16 else "32x32x16", "k_splits": splits,
+            "tail_tiles": tail, "tail_splits": tail_splits, "group_n": group_n, "peers_on_mfma": bool(mfma_peers),
+            "ragged": bool(ragged)}
 
 
 def reload_env() -> None:

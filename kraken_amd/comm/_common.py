@@ -6,7 +6,7 @@ from typing import Sequence
 
 import torch
 
-from .. import _lib
+from .. import _lib, _waits
 
 
 class PeerBuffers:
@@ -78,30 +78,57 @@ class PeerBuffers:
 
     def reduce_rmsnorm(self, rows, D, bias_ptr, bias_is_vector, w_ptr, eps, y_ptr, stream) -> int:
         lib = _lib.load()
-        ws = row_workspace(self.tensors[0].device, lib.kr_rmsnorm_workspace_bytes(self.W, rows, D))
+        dev = self.tensors[0].device
+        ws = row_workspace(dev, lib.kr_rmsnorm_workspace_bytes(self.W, rows, D))
         ws_ptr, ws_bytes = (ws.data_ptr(), ws.numel()) if ws is not None else (None, 0)
+        # a few long rows: their wavefronts meet in the workspace, a bounded wait that reports through
+        # the stream's status word like the flag waits of the overlap paths
+        status = _waits.new_status(dev) if ws is not None else None
         if self.stacked is not None:
-            return lib.kr_reduce_rmsnorm_ws_bf16(self.stacked.data_ptr(), self.W, self.stride, rows, D, bias_ptr,
-                                                 bias_is_vector, w_ptr, eps, y_ptr, ws_ptr, ws_bytes, stream)
-        return lib.kr_reduce_rmsnorm_ptrs_ws_bf16(self._table(0), self.W, rows, D, bias_ptr, bias_is_vector,
-                                                  w_ptr, eps, y_ptr, ws_ptr, ws_bytes, stream)
+            rc = lib.kr_reduce_rmsnorm_ws_bf16(self.stacked.data_ptr(), self.W, self.stride, rows, D, bias_ptr,
+                                               bias_is_vector, w_ptr, eps, y_ptr, ws_ptr, ws_bytes, _lib.ptr(status),
+                                               stream)
+        else:
+            rc = lib.kr_reduce_rmsnorm_ptrs_ws_bf16(self._table(0), self.W, rows, D, bias_ptr, bias_is_vector,
+                                                    w_ptr, eps, y_ptr, ws_ptr, ws_bytes, _lib.ptr(status), stream)
+        if status is not None and rc == 0:
+            # (the word is sticky and these calls take microseconds: mirroring it to the host now and
+            # then is enough to report a time-out, every call would cost more than the kernel)
+            _waits.watch(status, "reduce + RMSNorm of a few long rows (rows spread over many compute units)",
+                         min_interval_s=0.05)
+        return rc
 
 
-_row_workspaces: dict[tuple[int, int], torch.Tensor] = {}
+_row_workspaces: dict[tuple[int, int], tuple[torch.Tensor, torch.cuda.Stream]] = {}
 
 
 def row_workspace(dev: torch.device, nbytes: int) -> torch.Tensor | None:
-    """Workspace of the split-row RMSNorm kernel: one zero-initialised buffer per (device, stream),
-    so that calls on different streams never share one; the kernels keep it consistent afterwards."""
+    """Workspace of the split-row RMSNorm kernel: one zero-initialised buffer per (device, stream
+    that is current at the call), so that eager calls on different streams never share one; the
+    kernels keep it consistent afterwards.  A call that is captured into a graph bakes in the
+    workspace of the capture stream, whatever stream the graph is later replayed on: replays of
+    that graph must not overlap each other, other graphs captured on the same stream, or eager
+    calls on the capture stream (calls that share a workspace and overlap give NaN rows or wrong
+    ones).  After a reported time-out of the rows' exchange every workspace is zeroed again."""
     if nbytes <= 0:
         return None
-    key = (dev.index if dev.index is not None else torch.cuda.current_device(),
-           torch.cuda.current_stream(dev).cuda_stream)
-    ws = _row_workspaces.get(key)
-    if ws is None or ws.numel() < nbytes:
-        ws = torch.zeros(nbytes, dtype=torch.uint8, device=dev)
-        _row_workspaces[key] = ws
-    return ws
+    stream = torch.cuda.current_stream(dev)
+    key = (dev.index if dev.index is not None else torch.cuda.current_device(), stream.cuda_stream)
+    entry = _row_workspaces.get(key)
+    if entry is None or entry[0].numel() < nbytes:
+        entry = (torch.zeros(nbytes, dtype=torch.uint8, device=dev), stream)
+        _row_workspaces[key] = entry
+    return entry[0]
+
+
+def _zero_row_workspaces() -> None:
+    # after a time-out the slots of a workspace may carry tags that a later call would take for fresh ones
+    for ws, stream in _row_workspaces.values():
+        with torch.cuda.stream(stream):
+            ws.zero_()
+
+
+_waits.on_failure(_zero_row_workspaces)
 
 
 def check_stack(stacked: torch.Tensor | Sequence[torch.Tensor]) -> PeerBuffers:

@@ -500,6 +500,98 @@ static int static_scratch(void** out) {
     return KR_OK;
 }
 
+// ---- which kernel a call gets ----------------------------------------------------------------
+// One place decides it, for the launch and for kr_gemm_plan (which reports the decision).
+struct GemmPlan {
+    int tile;            // 256: LDS-DMA kernel (gemm_dtl.hip); 128: register-staged kernel (this file)
+    int mi16;            // 256x256 kernel: k loop on 16x16x32 blocks (else 32x32x16)
+    int peers_on_mfma;   // 256x256 kernel, 32x32x16 form: whole-band tiles add their peers on the matrix cores
+    int group_n;         // column panels per scheduling group
+    int tail_tiles;      // 256x256 kernel: tiles of the last partial round that are split ...
+    int tail_splits;     // ... into this many parts each
+    int splits;          // 128x128 kernel: workgroups per tile (split K loop), 1 = one pass
+};
+static GemmPlan plan_gemm(int64_t M, int64_t N, int64_t K, bool b_nt, int n_peers, int64_t band_rows, bool plain,
+                          bool has_workspace, int64_t workspace_bytes, bool has_gather, bool has_progress, bool flagged,
+                          bool dtl_ok) {
+    GemmPlan p{};
+    // Tile choice: the 256x256 tile of the LDS-DMA kernel (4 waves x 128x128) has the highest
+    // MFMA work per LDS/HBM byte; it needs K % 64 == 0 and a K loop long enough to amortise
+    // its epilogue.  Otherwise 128x128 tiles, two of which share a CU so that one
+    // tile's epilogue overlaps the other's MFMAs; they also win while all of them fit on the
+    // 256 CUs at once (512 tiles = 128 of the large ones): measured, the large tile is 15-30 %
+    // faster from 144 tiles on and 5-10 % slower at 128, for K from 1024 to 8192.
+    bool big = ((M + 255) / 256) * ((N + 255) / 256) > 128 && K >= 256;
+    // (few rows and a long K loop: the large tile again, with every tile's K loop split)
+    if (!big && has_workspace && !has_gather && whole_launch_split_pays(M, N, K, b_nt, plain)) {
+        int tail, ts;
+        tail_split_plan((M / 256) * (N / 256), K, &tail, &ts);
+        big = tail > 0 && gemm_dtl_tail_workspace_bytes(tail, ts) <= workspace_bytes;
+    }
+    // KRAKEN_AMD_GEMM_TILE=128|256 overrides the choice (testing and tuning)
+    if (env_switches().gemm_tile == 128) big = false;
+    if (env_switches().gemm_tile == 256) big = true;
+    const bool dtl = big && dtl_ok;
+    p.tile = dtl ? 256 : 128;
+    // KRAKEN_AMD_GEMM_PEERS=epilogue keeps the peers' partial sums out of the matrix cores
+    // (they are then added in the epilogue, where a non-finite value stays in its element)
+    p.peers_on_mfma = 1;
+    if (env_switches().gemm_peers >= 0) p.peers_on_mfma = env_switches().gemm_peers;
+    // MFMA block shape of the 256x256 kernel's k loop: 16x16x32 draws less power per flop than
+    // 32x32x16 and the chip is power-limited (5-10 % faster with warm operands; results agree to fp32 rounding).  It
+    // has no form that adds the peers on the matrix cores: its tiles add them in the epilogue,
+    // which costs little while the band is a small part of the rows (8192x8192x3584 with a band
+    // of 1024 rows: 367 -> 354 us) and much when every tile has peers (4096x8192x1024: 120 ->
+    // 146 us), so reduce-heavy calls keep 32x32x16.  KRAKEN_AMD_GEMM_MFMA=16|32 overrides.
+    p.mi16 = !(n_peers > 0 && band_rows * 2 >= M);
+    if (env_switches().gemm_mfma > 0) p.mi16 = env_switches().gemm_mfma == 16;
+    const int bm = p.tile;
+    const int64_t tiles_m = (M + bm - 1) / bm, tiles_n = (N + bm - 1) / bm;
+    // Column panels per scheduling group: the tiles an XCD runs at a time form a block that is
+    // group_n panels wide.  8 measured best for the compute-bound shapes; where most tiles also
+    // stream the peers' partial sums (HBM-bound), 16 lets neighbouring CUs read longer runs of
+    // the same rows at about the same time.
+    // (transposed-contiguous B: 4 measured 1-3 % ahead of 8 on 8192x3584x8192 and on the K = 16384
+    // shapes with N = 6656, level elsewhere; row-major B: 8 and 4 level)
+    p.group_n = (n_peers > 0 && band_rows * 2 >= M) ? 16 : (b_nt ? 4 : 8);
+    // Rows that arrive while the kernel runs: narrow groups, so that the range of tiles each XCD
+    // walks spans all row blocks in the order of their arrival (every XCD then starts on the
+    // local shard and waits little); with wide groups the XCDs that own the last blocks idle
+    // until those have arrived.
+    // The same for row bands that are flagged as they complete: every XCD then moves from band to
+    // band in the order of the destinations, and a band is complete once all eight have passed it
+    // (with wide groups every band would only be complete when the last group is).
+    if (flagged) p.group_n = (int)((tiles_n + kXcds - 1) / kXcds);
+    if (const int v = env_switches().gemm_group; v >= 1 && v <= 64) p.group_n = v;
+    // 256x256 kernel: the last partial round of tiles, split over the idle CUs (workspace given)
+    p.tail_tiles = 0;
+    p.tail_splits = 1;
+    if (dtl && has_workspace && !has_progress && M % 256 == 0 && N % 256 == 0) {
+        int tail, ts;
+        tail_split_plan(tiles_m * tiles_n, K, &tail, &ts);
+        if (tail > 0 && gemm_dtl_tail_workspace_bytes(tail, ts) <= workspace_bytes) {
+            p.tail_tiles = tail;
+            p.tail_splits = ts;
+        }
+    }
+    // Split K loop (128x128 kernel, workspace given): with few tiles most CUs would idle, so S
+    // workgroups share a tile's K loop and meet in the workspace.
+    p.splits = 1;
+    if (!dtl && has_workspace) {
+        p.splits = split_k_factor(tiles_m * tiles_n, K);
+        if (p.splits > 1 && split_k_workspace_bytes(M, N, p.splits) > workspace_bytes) p.splits = 1;
+    }
+    return p;
+}
+
+// Everything kr_gemm_reduce_noalloc_bf16 would otherwise do on its first call on a device: loads
+// the library's code for the current device (a lazily loaded code object is what allocates the
+// device memory of the scratch array) and looks the array up.
+extern "C" int kr_init(void) {
+    void* p = nullptr;
+    return static_scratch(&p);
+}
+
 // What the kernel exchanges with other streams while it runs (null pointer to gemm_reduce:
 // nothing): the arrival flags of the all-gather matmul (progress == nullptr: A is complete) and
 // the per-band counters of the producer GEMM (band_counter == nullptr: none).
@@ -543,6 +635,7 @@ static int gemm_reduce(const void* A, int64_t lda_m, int64_t lda_k, const void* 
     if (!aligned16(A) || !aligned16(B) || !aligned16(bias) || !aligned16(c_full) || !aligned16(out))
         return KR_ERR_ALIGNMENT;
     // (arguments are checked; a shape that is split now gets the library's own workspace)
+    if (static_ws && kr_gemm_workspace_bytes(M, N, K) > KR_STATIC_SCRATCH_BYTES) return KR_ERR_SCRATCH;
     if (static_ws && kr_gemm_workspace_bytes(M, N, K) > 0) {
         const int rc = static_scratch(&workspace);
         if (rc != KR_OK) return rc;
@@ -598,24 +691,11 @@ static int gemm_reduce(const void* A, int64_t lda_m, int64_t lda_k, const void* 
     g.out = out;
     g.out_is_fp32 = out_is_fp32;
 
-    // Tile choice: the 256x256 tile of the LDS-DMA kernel (4 waves x 128x128) has the highest
-    // MFMA work per LDS/HBM byte; it needs K % 64 == 0 and a K loop long enough to amortise
-    // its epilogue.  Otherwise 128x128 tiles, two of which share a CU so that one
-    // tile's epilogue overlaps the other's MFMAs; they also win while all of them fit on the
-    // 256 CUs at once (512 tiles = 128 of the large ones): measured, the large tile is 15-30 %
-    // faster from 144 tiles on and 5-10 % slower at 128, for K from 1024 to 8192.
-    bool big = ((M + 255) / 256) * ((N + 255) / 256) > 128 && K >= 256;
-    // (few rows and a long K loop: the large tile again, with every tile's K loop split)
-    if (!big && workspace != nullptr && gather == nullptr && whole_launch_split_pays(M, N, K, b_nt, n_peers == 0 && c_full == nullptr && bias == nullptr)) {
-        int tail, ts;
-        tail_split_plan((M / 256) * (N / 256), K, &tail, &ts);
-        big = tail > 0 && gemm_dtl_tail_workspace_bytes(tail, ts) <= workspace_bytes;
-    }
-    // KRAKEN_AMD_GEMM_TILE=128|256 overrides the choice (testing and tuning)
-    if (env_switches().gemm_tile == 128) big = false;
-    if (env_switches().gemm_tile == 256) big = true;
-    const bool dtl = big && gemm_dtl_supported(g) &&
-                     (g.a_local == nullptr || (int64_t)256 * g.lda_local * 2 < 0x7fffffffLL);
+    const GemmPlan plan = plan_gemm(M, N, K, b_nt, n_peers, band_rows, n_peers == 0 && c_full == nullptr && bias == nullptr,
+                                    workspace != nullptr, workspace_bytes, gather != nullptr, g.progress != nullptr,
+                                    g.progress != nullptr || g.band_counter != nullptr,
+                                    gemm_dtl_supported(g) && (g.a_local == nullptr || (int64_t)256 * g.lda_local * 2 < 0x7fffffffLL));
+    const bool dtl = plan.tile == 256;
     // The 128x128 kernel addresses a tile's operand panels with 32-bit byte offsets from the
     // panel's first row (through a 2 GiB buffer descriptor): row strides beyond that reach are
     // refused rather than read as zeros.
@@ -623,58 +703,23 @@ static int gemm_reduce(const void* A, int64_t lda_m, int64_t lda_k, const void* 
         const int64_t reach = std::max<int64_t>(std::max(lda_m, ldb), g.a_local != nullptr ? g.lda_local : 0);
         if ((128 * reach + std::max(K, N)) * 2 >= 0x7fffffffLL) return KR_ERR_LAYOUT;
     }
-    // KRAKEN_AMD_GEMM_PEERS=epilogue keeps the peers' partial sums out of the matrix cores
-    // (they are then added in the epilogue, where a non-finite value stays in its element)
-    g.peers_on_mfma = 1;
-    if (env_switches().gemm_peers >= 0) g.peers_on_mfma = env_switches().gemm_peers;
-    // MFMA block shape of the 256x256 kernel's k loop: 16x16x32 draws less power per flop than
-    // 32x32x16 and the chip is power-limited (5-10 % faster with warm operands; results agree to fp32 rounding).  It
-    // has no form that adds the peers on the matrix cores: its tiles add them in the epilogue,
-    // which costs little while the band is a small part of the rows (8192x8192x3584 with a band
-    // of 1024 rows: 367 -> 354 us) and much when every tile has peers (4096x8192x1024: 120 ->
-    // 146 us), so reduce-heavy calls keep 32x32x16.  KRAKEN_AMD_GEMM_MFMA=16|32 overrides.
-    g.mi16 = !(n_peers > 0 && band_rows * 2 >= M);
-    if (env_switches().gemm_mfma > 0) g.mi16 = env_switches().gemm_mfma == 16;
-    const int bm = dtl ? 256 : 128, bn = bm;
+    g.peers_on_mfma = plan.peers_on_mfma;
+    g.mi16 = plan.mi16;
+    const int bm = plan.tile, bn = bm;
     g.tiles_m = (int)((M + bm - 1) / bm);
     g.tiles_n = (int)((N + bn - 1) / bn);
     if ((int64_t)g.tiles_m * g.tiles_n > 0x7fffffffLL) return KR_ERR_BAD_DIM;
-    // Column panels per scheduling group: the tiles an XCD runs at a time form a block that is
-    // group_n panels wide.  8 measured best for the compute-bound shapes; where most tiles also
-    // stream the peers' partial sums (HBM-bound), 16 lets neighbouring CUs read longer runs of
-    // the same rows at about the same time.
-    // (transposed-contiguous B: 4 measured 1-3 % ahead of 8 on 8192x3584x8192 and on the K = 16384
-    // shapes with N = 6656, level elsewhere; row-major B: 8 and 4 level)
-    g.group_n = (n_peers > 0 && band_rows * 2 >= M) ? 16 : (b_nt ? 4 : 8);
-    // Rows that arrive while the kernel runs: narrow groups, so that the range of tiles each XCD
-    // walks spans all row blocks in the order of their arrival (every XCD then starts on the
-    // local shard and waits little); with wide groups the XCDs that own the last blocks idle
-    // until those have arrived.
-    // The same for row bands that are flagged as they complete: every XCD then moves from band to
-    // band in the order of the destinations, and a band is complete once all eight have passed it
-    // (with wide groups every band would only be complete when the last group is).
-    if (g.progress != nullptr || g.band_counter != nullptr) g.group_n = (g.tiles_n + kXcds - 1) / kXcds;
-    if (const int v = env_switches().gemm_group; v >= 1 && v <= 64) g.group_n = v;
-    // Split K loop (128x128 kernel, workspace given): with few tiles most CUs would idle, so S
-    // workgroups share a tile's K loop and meet in the workspace.
+    g.group_n = plan.group_n;
     g.k_splits = 1;
     g.split_out_stride = 0;
     g.tail_tiles = 0;
-    if (dtl && workspace != nullptr && g.progress == nullptr && M % 256 == 0 && N % 256 == 0) {
-        int tail, ts;
-        tail_split_plan((int64_t)g.tiles_m * g.tiles_n, K, &tail, &ts);
-        if (tail > 0 && gemm_dtl_tail_workspace_bytes(tail, ts) <= workspace_bytes) {
-            if (!aligned16(workspace)) return KR_ERR_ALIGNMENT;
-            g.tail_tiles = tail;
-            g.k_splits = ts;
-        }
+    if (plan.tail_tiles > 0) {
+        if (!aligned16(workspace)) return KR_ERR_ALIGNMENT;
+        g.tail_tiles = plan.tail_tiles;
+        g.k_splits = plan.tail_splits;
     }
-    int splits = 1;
-    if (!dtl && workspace != nullptr) {
-        splits = split_k_factor((int64_t)g.tiles_m * g.tiles_n, K);
-        if (splits > 1 && split_k_workspace_bytes(M, N, splits) > workspace_bytes) splits = 1;
-        if (splits > 1 && !aligned16(workspace)) return KR_ERR_ALIGNMENT;
-    }
+    const int splits = plan.splits;
+    if (splits > 1 && !aligned16(workspace)) return KR_ERR_ALIGNMENT;
     int64_t pt = tile_pivot / bm;
     g.pivot_tiles = (int)(((pt % g.tiles_m) + g.tiles_m) % g.tiles_m);
     const bool even = (M % bm == 0 && N % bn == 0 && K % BK == 0);
@@ -767,6 +812,32 @@ extern "C" int kr_gemm_producer_bf16(const void* A, int64_t lda_m, int64_t lda_k
                        0, ((int64_t)(rank + 1) % W) * (M / W), stream, &ps);
 }
 
+extern "C" int kr_gemm_plan(int64_t M, int64_t N, int64_t K, int b_transposed, int n_peers, int64_t band_rows,
+                            int has_bias, int has_c_full, int64_t workspace_bytes, int32_t plan[8]) {
+    if (plan == nullptr) return KR_ERR_NULL_POINTER;
+    if (M <= 0 || N <= 0 || K <= 0 || M > 0x7fffffffLL || N > 0x7fffffffLL || K > 0x7fffffffLL) return KR_ERR_BAD_DIM;
+    if (n_peers < 0 || n_peers >= KR_MAX_WORLD) return KR_ERR_WORLD_SIZE;
+    if (band_rows < 0 || band_rows > M) return KR_ERR_BAND;
+    // contiguous operands: the only other input of the choice is whether the 256-row panels stay
+    // within the 2 GiB reach of a buffer descriptor
+    GemmArgs g{};
+    g.K = (int)K;
+    g.lda = K;
+    g.ldb = b_transposed ? K : N;
+    const GemmPlan p = plan_gemm(M, N, K, b_transposed != 0, n_peers, band_rows, n_peers == 0 && !has_c_full && !has_bias,
+                                 workspace_bytes > 0, workspace_bytes, false, false, false, gemm_dtl_supported(g));
+    const bool whole_band_peers = p.tile == 256 && !p.mi16 && n_peers > 0 && p.peers_on_mfma != 0;
+    plan[0] = p.tile;
+    plan[1] = p.tile == 256 ? (p.mi16 ? 16 : 32) : 32;   // MFMA block rows: 16x16x32 or 32x32x16
+    plan[2] = p.splits;
+    plan[3] = p.tail_tiles;
+    plan[4] = p.tail_splits;
+    plan[5] = p.group_n;
+    plan[6] = whole_band_peers ? 1 : 0;
+    plan[7] = (M % p.tile != 0 || N % p.tile != 0) ? 1 : 0;
+    return KR_OK;
+}
+
 extern "C" int64_t kr_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K) {
     if (M <= 0 || N <= 0 || K <= 0) return 0;
     // the large-tile kernel (same rule as the launch; strides are not known here)
@@ -821,7 +892,6 @@ extern "C" int kr_gemm_reduce_noalloc_bf16(const void* A, int64_t lda_m, int64_t
                                            const void* bias, int64_t band_row0, int64_t band_rows,
                                            void* c_full, void* out, int out_is_fp32, int64_t tile_pivot,
                                            void* stream) {
-    if (kr_gemm_workspace_bytes(M, N, K) > KR_STATIC_SCRATCH_BYTES) return KR_ERR_SCRATCH;
     return gemm_reduce(A, lda_m, lda_k, B, ldb_k, ldb_n, M, N, K, peers, n_peers, nullptr, peers_stride, bias,
                        band_row0, band_rows, c_full, out, out_is_fp32, tile_pivot, stream, nullptr, nullptr, 0,
                        /*static_ws=*/true);

@@ -172,7 +172,10 @@ __global__ __launch_bounds__(kMaxThreads) void reduce_rmsnorm_kernel(
 // of the exchange).  All wavefronts of a row are resident together (the grid is at most
 // kSplitMaxWaves one-wave workgroups, dispatched in order), so the poll ends; it is bounded all
 // the same: after kSplitSpinLimit polls (seconds) the wavefront gives up and its piece of the row
-// is written as NaN.  Tags are 32 bits: a slot left by an earlier call could only be mistaken for
+// is written as NaN (and 1 + row goes to the caller's status word).  After such a time-out the
+// workspace is no longer consistent -- a wavefront of the failed call that starts after wavefront 0
+// gave up reads the new generation and leaves a slot that the next call takes for a fresh one -- so
+// it must be zeroed before it is used again.  Tags are 32 bits: a slot left by an earlier call could only be mistaken for
 // a fresh one if exactly 2^32 calls on the workspace lay between two uses of that slot.
 constexpr int kSplitSlots = 64;                       // wavefronts per row at most -> D <= 32768
 constexpr int kSplitMaxRows = 64;
@@ -185,7 +188,7 @@ template <class SRC, int WT, int BIAS>
 __global__ __launch_bounds__(kWave) void reduce_rmsnorm_split_kernel(
     const SRC src, int d_vec, int nw,
     const u32x4* __restrict__ bias, const u32x4* __restrict__ wgt, float eps, float inv_d,
-    u32x4* __restrict__ y, uint64_t* __restrict__ ws) {
+    u32x4* __restrict__ y, uint64_t* __restrict__ ws, int* __restrict__ status) {
     const int row = blockIdx.x / nw;
     const int piece = blockIdx.x - row * nw;
     const int lane = threadIdx.x;
@@ -232,8 +235,10 @@ __global__ __launch_bounds__(kWave) void reduce_rmsnorm_split_kernel(
     float total = 0.0f;
     const int part = (int)(uint32_t)v;
     for (int k = 0; k < nw; ++k) total += __builtin_bit_cast(float, __builtin_amdgcn_readlane(part, k));
-    // a row whose wavefronts did not meet within the bound comes out as NaN, not as a plausible wrong value
+    // a row whose wavefronts did not meet within the bound comes out as NaN, not as a plausible wrong
+    // value, and the caller's status word (if any) names it
     const float rstd = met ? __builtin_amdgcn_rsqf(total * inv_d + eps) : __builtin_nanf("");
+    if (!met && status != nullptr && lane == 0) __hip_atomic_store(status, 1 + row, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 
     if (c < d_vec) {
         float wf[8], o[8];
@@ -262,19 +267,19 @@ static bool row_split_pays(int W, int64_t rows, int64_t D) {
 
 template <class SRC, int WT>
 static hipError_t launch_split2(int mode, dim3 grid, hipStream_t st, const SRC& tab, int d_vec, int nw,
-                                const u32x4* bias, const u32x4* wgt, float eps, float inv_d, u32x4* y, uint64_t* ws) {
+                                const u32x4* bias, const u32x4* wgt, float eps, float inv_d, u32x4* y, uint64_t* ws, int* status) {
     switch (mode) {
         case kRowNoBias:
             hipLaunchKernelGGL((reduce_rmsnorm_split_kernel<SRC, WT, kRowNoBias>), grid, dim3(kWave), 0, st, tab, d_vec,
-                               nw, bias, wgt, eps, inv_d, y, ws);
+                               nw, bias, wgt, eps, inv_d, y, ws, status);
             break;
         case kRowFullBias:
             hipLaunchKernelGGL((reduce_rmsnorm_split_kernel<SRC, WT, kRowFullBias>), grid, dim3(kWave), 0, st, tab, d_vec,
-                               nw, bias, wgt, eps, inv_d, y, ws);
+                               nw, bias, wgt, eps, inv_d, y, ws, status);
             break;
         default:
             hipLaunchKernelGGL((reduce_rmsnorm_split_kernel<SRC, WT, kRowVecBias>), grid, dim3(kWave), 0, st, tab, d_vec,
-                               nw, bias, wgt, eps, inv_d, y, ws);
+                               nw, bias, wgt, eps, inv_d, y, ws, status);
             break;
     }
     return hipGetLastError();
@@ -282,7 +287,7 @@ static hipError_t launch_split2(int mode, dim3 grid, hipStream_t st, const SRC& 
 
 template <class SRC>
 static int launch_split(const SRC& tab, int W, int64_t rows, int64_t D, const void* bias, int mode, const void* w,
-                        float eps, void* y, void* workspace, void* stream) {
+                        float eps, void* y, void* workspace, int* status, void* stream) {
     const int d_vec = (int)(D / 8);
     const int nw = (d_vec + kWave - 1) / kWave;
     const dim3 grid((unsigned)(rows * nw));
@@ -291,10 +296,10 @@ static int launch_split(const SRC& tab, int W, int64_t rows, int64_t D, const vo
     const u32x4* wp = (const u32x4*)w;
     const float inv_d = 1.0f / (float)D;
     switch (W) {
-        case 1: return (int)launch_split2<SRC, 1>(mode, grid, st, tab, d_vec, nw, bp, wp, eps, inv_d, (u32x4*)y, (uint64_t*)workspace);
-        case 2: return (int)launch_split2<SRC, 2>(mode, grid, st, tab, d_vec, nw, bp, wp, eps, inv_d, (u32x4*)y, (uint64_t*)workspace);
-        case 4: return (int)launch_split2<SRC, 4>(mode, grid, st, tab, d_vec, nw, bp, wp, eps, inv_d, (u32x4*)y, (uint64_t*)workspace);
-        default: return (int)launch_split2<SRC, 8>(mode, grid, st, tab, d_vec, nw, bp, wp, eps, inv_d, (u32x4*)y, (uint64_t*)workspace);
+        case 1: return (int)launch_split2<SRC, 1>(mode, grid, st, tab, d_vec, nw, bp, wp, eps, inv_d, (u32x4*)y, (uint64_t*)workspace, status);
+        case 2: return (int)launch_split2<SRC, 2>(mode, grid, st, tab, d_vec, nw, bp, wp, eps, inv_d, (u32x4*)y, (uint64_t*)workspace, status);
+        case 4: return (int)launch_split2<SRC, 4>(mode, grid, st, tab, d_vec, nw, bp, wp, eps, inv_d, (u32x4*)y, (uint64_t*)workspace, status);
+        default: return (int)launch_split2<SRC, 8>(mode, grid, st, tab, d_vec, nw, bp, wp, eps, inv_d, (u32x4*)y, (uint64_t*)workspace, status);
     }
 }
 
@@ -352,9 +357,9 @@ static void row_geometry(int d_vec, int* threads, int* vpt) {
 template <class SRC>
 static int launch_rows(const SRC& tab, int W, int64_t rows, int64_t D, const void* bias,
                        int mode, const void* w, float eps, void* y, void* stream,
-                       void* workspace = nullptr, int64_t workspace_bytes = 0) {
+                       void* workspace = nullptr, int64_t workspace_bytes = 0, int* status = nullptr) {
     if (workspace != nullptr && workspace_bytes >= kSplitWorkspaceBytes && row_split_pays(W, rows, D))
-        return launch_split(tab, W, rows, D, bias, mode, w, eps, y, workspace, stream);
+        return launch_split(tab, W, rows, D, bias, mode, w, eps, y, workspace, status, stream);
     int threads, vpt;
     const int d_vec = (int)(D / 8);
     row_geometry(d_vec, &threads, &vpt);
@@ -408,40 +413,42 @@ extern "C" int64_t kr_rmsnorm_workspace_bytes(int W, int64_t rows, int64_t D) {
 
 extern "C" int kr_reduce_rmsnorm_ws_bf16(const void* stack, int W, int64_t slice_stride, int64_t rows, int64_t D,
                                          const void* bias, int bias_is_vector, const void* w, float eps, void* y,
-                                         void* workspace, int64_t workspace_bytes, void* stream) {
+                                         void* workspace, int64_t workspace_bytes, int32_t* status, void* stream) {
     if (W >= 1 && W <= KR_MAX_WORLD && slice_stride < 0) return KR_ERR_BAD_DIM;
     int rc = check_rows(W, rows, D, bias, w, y);
     if (rc != KR_OK || rows == 0) return rc;
     if (stack == nullptr) return KR_ERR_NULL_POINTER;
     if (!aligned16(stack) || slice_stride % 8 != 0 || !aligned16(workspace)) return KR_ERR_ALIGNMENT;
+    if ((reinterpret_cast<uintptr_t>(status) & 3u) != 0) return KR_ERR_ALIGNMENT;
     const int mode = bias == nullptr ? kRowNoBias : (bias_is_vector ? kRowVecBias : kRowFullBias);
     const StackedPeers src{(const u32x4*)stack, slice_stride / 8};
-    return launch_rows(src, W, rows, D, bias, mode, w, eps, y, stream, workspace, workspace_bytes);
+    return launch_rows(src, W, rows, D, bias, mode, w, eps, y, stream, workspace, workspace_bytes, status);
 }
 
 extern "C" int kr_reduce_rmsnorm_bf16(const void* stack, int W, int64_t slice_stride, int64_t rows, int64_t D,
                                       const void* bias, int bias_is_vector, const void* w, float eps, void* y,
                                       void* stream) {
     return kr_reduce_rmsnorm_ws_bf16(stack, W, slice_stride, rows, D, bias, bias_is_vector, w, eps, y, nullptr, 0,
-                                     stream);
+                                     nullptr, stream);
 }
 
 extern "C" int kr_reduce_rmsnorm_ptrs_ws_bf16(const void* const* bufs, int W, int64_t rows, int64_t D,
                                               const void* bias, int bias_is_vector, const void* w, float eps,
-                                              void* y, void* workspace, int64_t workspace_bytes, void* stream) {
+                                              void* y, void* workspace, int64_t workspace_bytes, int32_t* status,
+                                              void* stream) {
     int rc = check_rows(W, rows, D, bias, w, y);
     if (rc != KR_OK || rows == 0) return rc;
     PeerTab tab;
     if ((rc = peer_tab_from_ptrs(tab, bufs, W)) != KR_OK) return rc;
-    if (!aligned16(workspace)) return KR_ERR_ALIGNMENT;
+    if (!aligned16(workspace) || (reinterpret_cast<uintptr_t>(status) & 3u) != 0) return KR_ERR_ALIGNMENT;
     const int mode = bias == nullptr ? kRowNoBias : (bias_is_vector ? kRowVecBias : kRowFullBias);
-    return launch_rows(tab, W, rows, D, bias, mode, w, eps, y, stream, workspace, workspace_bytes);
+    return launch_rows(tab, W, rows, D, bias, mode, w, eps, y, stream, workspace, workspace_bytes, status);
 }
 
 extern "C" int kr_reduce_rmsnorm_ptrs_bf16(const void* const* bufs, int W, int64_t rows, int64_t D,
                                            const void* bias, int bias_is_vector, const void* w, float eps,
                                            void* y, void* stream) {
-    return kr_reduce_rmsnorm_ptrs_ws_bf16(bufs, W, rows, D, bias, bias_is_vector, w, eps, y, nullptr, 0, stream);
+    return kr_reduce_rmsnorm_ptrs_ws_bf16(bufs, W, rows, D, bias, bias_is_vector, w, eps, y, nullptr, 0, nullptr, stream);
 }
 
 extern "C" int kr_rmsnorm_bf16(const void* x, const void* w, float eps, int64_t rows, int64_t D, void* y,

@@ -111,6 +111,7 @@ def all_gather_matmul(
 
     assert K % 8 == 0, "K must be a multiple of 8"
     assert m % splits == 0, "splits_per_rank must divide the rows of a shard"
+    _waits.check()      # an earlier call's failed wait is reported before anything of this call is enqueued
     if a_out is None:
         a_out = torch.empty((M, K), dtype=torch.bfloat16, device=dev)
     else:
@@ -123,7 +124,6 @@ def all_gather_matmul(
                                                         copy_engine=kwargs.get("copy_engine", False))
     configs = {"RANK": rank, "WORLD_SIZE": W, "SPLITS_PER_RANK": splits,
                "wait_limit_us": kwargs.get("wait_limit_us", 0)}
-    _waits.check()
     status = kwargs.get("status")
     own_status = status is None
     if own_status:

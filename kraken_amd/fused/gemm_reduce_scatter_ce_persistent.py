@@ -172,6 +172,7 @@ def gemm_reduce_scatter_ce_persistent(
     P, _ = _gemm.check_peers(peers, m_per_rank, N)
     assert P == world_size - 1
     dev = _lib.require_device(a, b)
+    _waits.check()      # an earlier call's failed wait is reported before anything of this call is enqueued
     gemm_out = torch.empty((M, N), dtype=a.dtype, device=dev)
     scatter_out = torch.empty((world_size, m_per_rank, N), dtype=a.dtype, device=dev)
     output = torch.empty((m_per_rank, N), dtype=a.dtype, device=dev)

@@ -75,12 +75,14 @@ def test_rmsnorm_workspace_entries(lib, monkeypatch):
     assert q(8, 256, 4096) == 0 and q(8, 16, 1024) == 0 and q(3, 16, 8192) == 0 and q(8, 128, 8192) == 0
     assert q(8, 16, 8190) == 0 and q(8, 0, 8192) == 0 and q(8, 2, 65536) == 0
     f = lib.kr_reduce_rmsnorm_ws_bf16
-    assert f(FAKE, 8, 8192 * 16, 16, 8192, None, 0, FAKE, 1e-5, FAKE, FAKE + 8, need, None) == _lib.KR_ERR_ALIGNMENT
-    assert f(FAKE, 8, 8192 * 16, 16, 8196, None, 0, FAKE, 1e-5, FAKE, FAKE, need, None) == _lib.KR_ERR_NUMEL_MOD8
-    assert f(None, 8, 8192 * 16, 16, 8192, None, 0, FAKE, 1e-5, FAKE, FAKE, need, None) == _lib.KR_ERR_NULL_POINTER
-    assert f(FAKE, 8, 8192 * 16, 0, 8192, None, 0, FAKE, 1e-5, FAKE, FAKE, need, None) == 0
+    assert f(FAKE, 8, 8192 * 16, 16, 8192, None, 0, FAKE, 1e-5, FAKE, FAKE + 8, need, None, None) == _lib.KR_ERR_ALIGNMENT
+    assert f(FAKE, 8, 8192 * 16, 16, 8196, None, 0, FAKE, 1e-5, FAKE, FAKE, need, None, None) == _lib.KR_ERR_NUMEL_MOD8
+    assert f(None, 8, 8192 * 16, 16, 8192, None, 0, FAKE, 1e-5, FAKE, FAKE, need, None, None) == _lib.KR_ERR_NULL_POINTER
+    # the status word of the bounded exchange: 4-byte aligned or NULL
+    assert f(FAKE, 8, 8192 * 16, 16, 8192, None, 0, FAKE, 1e-5, FAKE, FAKE, need, FAKE + 2, None) == _lib.KR_ERR_ALIGNMENT
+    assert f(FAKE, 8, 8192 * 16, 0, 8192, None, 0, FAKE, 1e-5, FAKE, FAKE, need, FAKE, None) == 0
     g = lib.kr_reduce_rmsnorm_ptrs_ws_bf16
-    assert g(None, 8, 16, 8192, None, 0, FAKE, 1e-5, FAKE, FAKE, need, None) == _lib.KR_ERR_NULL_POINTER
+    assert g(None, 8, 16, 8192, None, 0, FAKE, 1e-5, FAKE, FAKE, need, None, None) == _lib.KR_ERR_NULL_POINTER
     monkeypatch.setenv("KRAKEN_AMD_ROW_SPLIT", "0")
     assert q(8, 16, 8192) == 0
     monkeypatch.setenv("KRAKEN_AMD_ROW_SPLIT", "1")
@@ -282,7 +284,55 @@ def test_gemm_noalloc_entry_checks_arguments_first(lib, monkeypatch):
     assert lib.kr_gemm_workspace_bytes(1024, 2048, 4096) == 16 * 1024 * 2048 * 4 > (64 << 20)
     assert f(FAKE, 4096, 1, FAKE, 2048, 1, 1024, 2048, 4096, None, 0, 0, None, 0, 1024, None, FAKE, 0, 0,
              None) == _lib.KR_ERR_SCRATCH
+    # an oversize shape with a bad argument reports the argument, as every other entry point would
+    assert f(None, 4096, 1, FAKE, 2048, 1, 1024, 2048, 4096, None, 0, 0, None, 0, 1024, None, FAKE, 0, 0,
+             None) == _lib.KR_ERR_NULL_POINTER
+    assert f(FAKE + 2, 4096, 1, FAKE, 2048, 1, 1024, 2048, 4096, None, 0, 0, None, 0, 1024, None, FAKE, 0, 0,
+             None) == _lib.KR_ERR_ALIGNMENT
+    assert f(FAKE, 4096, 2, FAKE, 2048, 1, 1024, 2048, 4096, None, 0, 0, None, 0, 1024, None, FAKE, 0, 0,
+             None) == _lib.KR_ERR_LAYOUT
     assert "scratch" in _lib.strerror(_lib.KR_ERR_SCRATCH)
+
+
+def test_gemm_plan_reports_the_dispatch(lib, monkeypatch):
+    """kr_gemm_plan names the kernel a shape gets, by the rule the launch itself uses."""
+    p = _lib.gemm_plan(8192, 8192, 3584, False, 7, 1024, False, True)        # GEMM + reduce-scatter shape
+    assert p["kernel"] == "gemm_dtl16_kernel" and p["tile"] == 256 and p["mfma"] == "16x16x32" and not p["peers_on_mfma"]
+    p = _lib.gemm_plan(4096, 8192, 1024, False, 7, 4096, True, False)        # every tile streams peers
+    assert p["kernel"] == "gemm_dtl_kernel" and p["mfma"] == "32x32x16" and p["peers_on_mfma"] and p["group_n"] == 16
+    p = _lib.gemm_plan(8192, 3584, 8192, True)                               # all-gather matmul shape
+    assert p["kernel"] == "gemm_dtl16_kernel" and p["group_n"] == 4 and p["tail_tiles"] == 0
+    p = _lib.gemm_plan(256, 256, 100 * 8, False)                             # K not a multiple of 64
+    assert p["kernel"] == "gemm_reduce_kernel" and p["tile"] == 128 and p["k_splits"] == 1
+    need = lib.kr_gemm_workspace_bytes(128, 6656, 4096)
+    p = _lib.gemm_plan(128, 6656, 4096, False, workspace_bytes=need)         # few tiles: split K loop
+    assert p["tile"] == 128 and p["k_splits"] > 1
+    assert _lib.gemm_plan(128, 6656, 4096, False)["k_splits"] == 1           # no workspace, no split
+    p = _lib.gemm_plan(4352, 4096, 8192, False, workspace_bytes=1 << 30)     # 272 tiles: 16 tail tiles split
+    assert p["tile"] == 256 and p["tail_tiles"] == 16 and p["tail_splits"] == 8
+    assert _lib.gemm_plan(300, 8192 + 8, 4096, False)["ragged"]
+    plan = (ctypes.c_int32 * 8)()
+    assert lib.kr_gemm_plan(0, 64, 64, 0, 0, 0, 0, 0, 0, plan) == _lib.KR_ERR_BAD_DIM
+    assert lib.kr_gemm_plan(64, 64, 64, 0, 16, 0, 0, 0, 0, plan) == _lib.KR_ERR_WORLD_SIZE
+    assert lib.kr_gemm_plan(64, 64, 64, 0, 0, 65, 0, 0, 0, plan) == _lib.KR_ERR_BAND
+    assert lib.kr_gemm_plan(64, 64, 64, 0, 0, 0, 0, 0, 0, None) == _lib.KR_ERR_NULL_POINTER
+    monkeypatch.setenv("KRAKEN_AMD_GEMM_MFMA", "32")
+    _lib.reload_env()
+    try:
+        assert _lib.gemm_plan(8192, 3584, 8192, True)["kernel"] == "gemm_dtl_kernel"
+    finally:
+        monkeypatch.delenv("KRAKEN_AMD_GEMM_MFMA")
+        _lib.reload_env()
+
+
+def test_probe_argument_errors(lib):
+    assert lib.kr_probe_read(FAKE, 24, None, None) == _lib.KR_ERR_NUMEL_MOD8
+    assert lib.kr_probe_read(None, 32, None, None) == _lib.KR_ERR_NULL_POINTER
+    assert lib.kr_probe_read(FAKE + 4, 32, None, None) == _lib.KR_ERR_ALIGNMENT
+    assert lib.kr_probe_read(None, 0, None, None) == 0
+    assert lib.kr_probe_copy(FAKE, None, 32, None) == _lib.KR_ERR_NULL_POINTER
+    assert lib.kr_probe_copy(FAKE, FAKE + 8, 32, None) == _lib.KR_ERR_ALIGNMENT
+    assert lib.kr_probe_copy(None, None, 0, None) == 0
 
 
 def test_striped_share_numel(lib):

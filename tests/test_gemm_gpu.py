@@ -455,6 +455,17 @@ def test_bounded_waits_without_a_status_do_not_fail_silently(dev):
         _waits.check(block=True)
     assert time.perf_counter() - t0 < 0.1                                 # one limit, not eight
     _waits.check(block=True)                                              # reported once
+    # two failing calls before anybody looks: both are named (the second gives up at once: the
+    # stream's word is still set when its waits start)
+    t0 = time.perf_counter()
+    copy_engine_scatter(inp, outs, never, rank=0, wait_limit_us=20000)
+    copy_engine_scatter(inp, outs, never, rank=0, wait_limit_us=20000)
+    with pytest.raises(KrakenAmdError) as both:
+        _waits.check(block=True)
+    assert str(both.value).count("copy_engine_scatter") == 2
+    assert time.perf_counter() - t0 < 0.1
+    _waits.check(block=True)
+    assert _waits.new_status(dev).item() == 0                             # cleared by the report
     # the all-gather matmul with chunks that never arrive (no copies are enqueued for this call)
     from kraken_amd.fused.all_gather_matmul import _matmul_w_progress
     m, K, Nn = 64, 128, 256

@@ -200,8 +200,9 @@ def test_split_rows_share_one_workspace_across_shapes_and_calls(dev, monkeypatch
 
 
 def test_split_rows_replay_from_a_graph(dev):
-    """Captured once, replayed with eager calls (which advance the rows' generations) in between:
-    every replay gives the eager bits."""
+    """Captured once, replayed with eager calls on the capture stream in between (they use the
+    workspace the graph has baked in and advance its rows' generations): every replay gives the
+    eager bits."""
     W, rows, D = 8, 16, 8192
     assert _split_used(W, rows, D)
     stack = orc.make_stack(W, (rows, D), seed0=42).to(dev)
@@ -221,8 +222,30 @@ def test_split_rows_replay_from_a_graph(dev):
                 fused.one_shot_all_reduce_bias_rms_norm(stack, None, bias, w, yg)
     for rep in range(3):
         yg.zero_()
-        fused.one_shot_all_reduce_bias_rms_norm(stack, None, bias, w, y)       # eager work between the replays
+        y.zero_()
         torch.cuda.synchronize()
+        with torch.cuda.stream(side):                                              # eager work between the replays,
+            fused.one_shot_all_reduce_bias_rms_norm(stack, None, bias, w, y)       # on the graph's workspace
+        torch.cuda.synchronize()
+        assert torch.equal(y, eager)
         g.replay()
         torch.cuda.synchronize()
         assert torch.equal(yg, eager)
+
+
+def test_split_rows_report_through_the_status_word(dev):
+    """The exchange of a row's wavefronts is a bounded wait like the flag waits: the wrapper hands the
+    kernel the stream's status word and registers it (rate-limited); a normal call leaves it at zero
+    and check(block=True) has nothing to raise."""
+    from kraken_amd import _waits
+    W, rows, D = 8, 16, 8192
+    assert _split_used(W, rows, D)
+    stack = orc.make_stack(W, (rows, D), seed0=3).to(dev)
+    bias, w = (t.to(dev) for t in orc.make_bias_weight(D, 3))
+    y = torch.empty(rows, D, dtype=BF16, device=dev)
+    _waits.check(block=True)
+    for _ in range(20):
+        fused.one_shot_all_reduce_bias_rms_norm(stack, None, bias, w, y)
+    assert _waits.new_status(dev).item() == 0
+    _waits.check(block=True)
+    assert len(_waits._pending) == 0
