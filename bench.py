@@ -19,8 +19,11 @@ iteration, median): W untimed warm-up steps, then the same workload for a
 fixed time (SETTLE_MS of launches, so that clocks and power state do not
 depend on what ran before), then exactly K steps between two device
 synchronisations with an event recorded on the launch stream before each
-step and after the last; the median of the K intervals is the kernel time
-the roofline figure uses, minimum and maximum are reported beside it.
+interval and after the last (an interval is one step for the GEMMs and as many
+steps as last 0.25 ms for shorter kernels, since an event between two launches
+costs about 2 us that would be charged to the kernel); the median of the
+intervals is the kernel time the roofline figure uses, minimum and maximum are
+reported beside it.
 Workloads of a few microseconds are replayed from a HIP graph of G launches
 instead (the host cannot enqueue them as fast as the GPU retires them): R
 replays, each between its own pair of events, median of replay / G.  Every
@@ -661,25 +664,48 @@ def time_gpu_graph(step, steps, warmup, nsets=1, replays=GRAPH_REPLAYS, settle_m
     return (t1 - t0) * 1e3 / (replays * G), _stats(per), replays * G
 
 
+MIN_INTERVAL_MS = 0.25           # an event interval of the eager protocol covers at least this much GPU time
+
+
 def time_gpu_eager(step, steps, warmup, settle_ms=SETTLE_MS):
-    """Exactly `steps` launches between two synchronisations, an event on the launch stream in
-    front of each and behind the last: (wall ms per step, statistics of the `steps` intervals)."""
+    """Exactly `steps` launches between two synchronisations, with events on the launch stream
+    that cut them into intervals: (wall ms per step, statistics of interval / its launches, steps).
+
+    An event between two launches costs about 2 us of GPU time on this machine (the launches no
+    longer run back to back), which would be charged to the kernel: an interval therefore covers
+    as many launches as it takes to last MIN_INTERVAL_MS -- one for the GEMMs, five for a 50 us
+    kernel -- so that the markers stay below one percent of what they bracket.
+    """
     import torch
 
     for i in range(warmup):
         step(i)
     _settle(lambda n: [step(warmup + k) for k in range(10)], settle_ms)
-    evs = [torch.cuda.Event(enable_timing=True) for _ in range(steps + 1)]
+    a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    a.record()
+    for k in range(10):
+        step(warmup + k)
+    b.record()
+    torch.cuda.synchronize()
+    est_ms = a.elapsed_time(b) / 10
+    stride = max(1, min(steps, int(-(-MIN_INTERVAL_MS // est_ms))))
+    marks = list(range(0, steps, stride)) + [steps]          # an event in front of these steps, and one at the end
+    evs = [torch.cuda.Event(enable_timing=True) for _ in marks]
     torch.cuda.synchronize()
     t0 = time.perf_counter()
-    evs[0].record()                      # on the current stream = the stream the kernels go to
+    nxt = 0
     for i in range(steps):
+        if i == marks[nxt]:
+            evs[nxt].record()            # on the current stream = the stream the kernels go to
+            nxt += 1
         step(warmup + i)
-        evs[i + 1].record()
+    evs[nxt].record()
     torch.cuda.synchronize()
     t1 = time.perf_counter()
-    per = [evs[i].elapsed_time(evs[i + 1]) for i in range(steps)]
-    return (t1 - t0) * 1e3 / steps, _stats(per), steps
+    per = [evs[j].elapsed_time(evs[j + 1]) / (marks[j + 1] - marks[j]) for j in range(len(marks) - 1)]
+    st = _stats(per)
+    st["launches_per_interval"] = stride
+    return (t1 - t0) * 1e3 / steps, st, steps
 
 
 def time_gpu(wl, steps, warmup):
@@ -782,7 +808,7 @@ def measure_gpu(wl, steps, warmup, dev, floors=False):
         "hbm_frac": wl.bytes / (ev_ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
         "bound": wl.bound,
         "timing": (f"hip graph of {timed // st['n']} launches, median of {st['n']} replays" if wl.use_graph
-                   else f"eager launches, median of {st['n']} per-step event intervals"),
+                   else f"eager launches, median of {st['n']} event intervals of {st['launches_per_interval']} launch(es)"),
         "algorithmic_bytes": wl.bytes,
         "traffic": traffic[0],
         "traffic_profiled_at": traffic[1],
