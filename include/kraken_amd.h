@@ -187,14 +187,15 @@ int kr_rmsnorm_bf16(const void* x, const void* w, float eps, int64_t rows, int64
  * bf16 result, tiles whose peers are added in the epilogue round the product
  * to bf16 before the sum, as gemm_reduce_scatter_fused.py:72 does.
  * Non-finite input: for shapes the 256x256 kernel takes (more than 128 tiles
- * of 256x256, K % 64 == 0) and a band of at least half the rows, the peers of
- * tiles lying wholly in the band are added on the matrix cores, where an
- * Inf/NaN in a peer also turns the rest of the aligned 32-column block of its
- * row into NaN.  This default DEVIATES from the reference, whose epilogue adds the
- * peers element by element (gemm_one_shot_all_reduce_fused.py:85-92) and so keeps a
- * non-finite value in its own element; finite inputs give the same results either
- * way.  KRAKEN_AMD_GEMM_PEERS=epilogue in the environment selects the reference's
- * behaviour (as calls with a smaller band, and the 16x16x32 form, always have).
+ * of 256x256, K % 64 == 0), the peers of tiles lying wholly in the band are added
+ * on the matrix cores, where an Inf/NaN in a peer also turns the rest of the
+ * aligned 16-column block of its row into NaN (32 columns with
+ * KRAKEN_AMD_GEMM_MFMA=32).  This default DEVIATES from the reference, whose
+ * epilogue adds the peers element by element
+ * (gemm_one_shot_all_reduce_fused.py:85-92) and so keeps a non-finite value in its
+ * own element; finite inputs give the same results either way.
+ * KRAKEN_AMD_GEMM_PEERS=epilogue in the environment selects the reference's
+ * behaviour.
  *
  * Replaces
  *   kraken/fused/gemm_one_shot_all_reduce_fused.py:56-99   (band = all rows)

@@ -537,13 +537,10 @@ static GemmPlan plan_gemm(int64_t M, int64_t N, int64_t K, bool b_nt, int n_peer
     // (they are then added in the epilogue, where a non-finite value stays in its element)
     p.peers_on_mfma = 1;
     if (env_switches().gemm_peers >= 0) p.peers_on_mfma = env_switches().gemm_peers;
-    // MFMA block shape of the 256x256 kernel's k loop: 16x16x32 draws less power per flop than
-    // 32x32x16 and the chip is power-limited (5-10 % faster with warm operands; results agree to fp32 rounding).  It
-    // has no form that adds the peers on the matrix cores: its tiles add them in the epilogue,
-    // which costs little while the band is a small part of the rows (8192x8192x3584 with a band
-    // of 1024 rows: 367 -> 354 us) and much when every tile has peers (4096x8192x1024: 120 ->
-    // 146 us), so reduce-heavy calls keep 32x32x16.  KRAKEN_AMD_GEMM_MFMA=16|32 overrides.
-    p.mi16 = !(n_peers > 0 && band_rows * 2 >= M);
+    // MFMA block shape of the 256x256 kernel: 16x16x32 draws less power per flop than 32x32x16 and
+    // the chip is power-limited (k loop 5-10 % faster with warm operands; results agree to fp32
+    // rounding), and its peer phase takes two peers per MFMA.  KRAKEN_AMD_GEMM_MFMA=16|32 overrides.
+    p.mi16 = 1;
     if (env_switches().gemm_mfma > 0) p.mi16 = env_switches().gemm_mfma == 16;
     const int bm = p.tile;
     const int64_t tiles_m = (M + bm - 1) / bm, tiles_n = (N + bm - 1) / bm;
@@ -826,7 +823,7 @@ extern "C" int kr_gemm_plan(int64_t M, int64_t N, int64_t K, int b_transposed, i
     g.ldb = b_transposed ? K : N;
     const GemmPlan p = plan_gemm(M, N, K, b_transposed != 0, n_peers, band_rows, n_peers == 0 && !has_c_full && !has_bias,
                                  workspace_bytes > 0, workspace_bytes, false, false, false, gemm_dtl_supported(g));
-    const bool whole_band_peers = p.tile == 256 && !p.mi16 && n_peers > 0 && p.peers_on_mfma != 0;
+    const bool whole_band_peers = p.tile == 256 && n_peers > 0 && p.peers_on_mfma != 0;
     plan[0] = p.tile;
     plan[1] = p.tile == 256 ? (p.mi16 ? 16 : 32) : 32;   // MFMA block rows: 16x16x32 or 32x32x16
     plan[2] = p.splits;

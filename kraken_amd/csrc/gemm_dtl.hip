@@ -65,8 +65,7 @@ constexpr int kLgkm0 = 0xc07f;   // s_waitcnt lgkmcnt(0) only
 // MI16: the k loop uses v_mfma_f32_16x16x32_bf16 (8 x 8 blocks of 16 x 16 per wave) instead of
 // 32x32x16 (4 x 4 blocks of 32 x 32): same operand traffic, but the matrix cores draw less power
 // per flop with it (under the power limit, matrix-core-only loops on random operands sustain
-// 2.04 PFLOP/s with 16x16x32 against 1.62 with 32x32x16).  No peers on the matrix cores in this
-// form.
+// 2.04 PFLOP/s with 16x16x32 against 1.62 with 32x32x16).
 template <bool B_NT, bool PEERS_FIRST, bool SPLIT = false, bool RAGGED = false, bool MI16 = false>
 __device__ __forceinline__ void gemm_dtl_tile(const GemmArgs& g, unsigned char* smem) {
     // Nothing is outstanding at kernel entry; saying so keeps the compiler's own wait-count
@@ -274,7 +273,7 @@ __device__ __forceinline__ void gemm_dtl_tile(const GemmArgs& g, unsigned char* 
     const int band_lo = g.band_row0;
     const bool full_tile = !RAGGED || (m0 + BM <= g.M && n0 + BN <= g.N);
     const bool tile_in_band = full_tile && m0 >= band_lo && m0 + BM <= band_lo + g.band_rows;
-    const bool mfma_peers = !SPLIT && !MI16 && g.peers_on_mfma && g.n_peers > 0 && tile_in_band;
+    const bool mfma_peers = !SPLIT && g.peers_on_mfma && g.n_peers > 0 && tile_in_band;
     const bool bias_in_acc = !SPLIT && g.bias != nullptr && tile_in_band && (g.n_peers == 0 || mfma_peers);
     f32x16 acc[TM][TN];
     {
@@ -408,6 +407,92 @@ __device__ __forceinline__ void gemm_dtl_tile(const GemmArgs& g, unsigned char* 
         __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));
         __syncthreads();   // the ring is handed on (k loop or epilogue patches of other waves)
     };
+    // The same on 16x16x32 blocks, where one MFMA takes the partial sums of TWO peers: with
+    //   Y[m][k] = P_a[m][16j + k] (k < 16),  P_b[m][16j + k - 16] (k >= 16)   and   X[n][k] = (k % 16 == n),
+    // acc16[n][m] += sum_{k<32} X[n][k] * Y[m][k] = P_a[m][16j + n] + P_b[m][16j + n].  The operand wants, per
+    // lane, 8 consecutive columns of one row: lanes 0..31 take them from peer a, lanes 32..63 from
+    // peer b.  An item is a pair's 16 rows x 128 columns of this wave (rows 0..15 of the stage: peer
+    // a, rows 16..31: peer b; 8 KiB, eight LDS-DMA loads); half as many MFMA cycles per peer as the
+    // 32x32x16 form.  An odd peer count repeats the last peer as b and masks it in X (a product
+    // 0 * finite adds nothing).
+    auto peer_phase16 = [&]() __attribute__((always_inline)) {
+        constexpr int kItemLoads = 8;
+        constexpr int kItemBytes = kItemLoads * 1024;
+        constexpr int kAhead = 4;
+        constexpr int kSlabs = 2 * TM;         // 16-row slabs of the wave
+        static_assert(kSlabs % kAhead == 0 && kAhead * kItemBytes * WM * WN <= LDS_BYTES, "peer stages must fit in the ring");
+        typedef short s16x8 __attribute__((ext_vector_type(8)));
+        bf16x8 xsel[2];   // [0]: both peers of the pair, [1]: peer a only
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            s16x8 x;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                const int k = 8 * (lane >> 4) + e;
+                x[e] = ((k & 15) == (lane & 15) && (h == 0 || k < 16)) ? (short)0x3f80 : (short)0;
+            }
+            xsel[h] = __builtin_bit_cast(bf16x8, x);
+        }
+        const uint32_t region = (uint32_t)wave * (kAhead * kItemBytes);
+        // load r of an item fills stage rows 4r .. 4r+3 (r < 4: peer a, else peer b): lane l -> row
+        // 4(r % 4) + l/16 of the slab, piece slot l%16 holds piece slot ^ row
+        uint32_t pvoff[4];
+#pragma unroll
+        for (int b = 0; b < 4; ++b) {
+            const int row = 4 * b + (lane >> 4);
+            pvoff[b] = (uint32_t)(((int64_t)row * g.N + (((lane & 15) ^ row) << 3)) * 2);
+        }
+        // fragment of column block bj: lane l -> stage row l%16 + 16(l/32), piece 2 bj + (l/16)%2
+        uint32_t pa[2 * TN];
+#pragma unroll
+        for (int bj = 0; bj < 2 * TN; ++bj) {
+            const int row = (lane & 15) + 16 * (lane >> 5);
+            pa[bj] = region + (uint32_t)(row * 256 + (((2 * bj + ((lane >> 4) & 1)) ^ (row & 15)) << 4));
+        }
+        const int n_pairs = (g.n_peers + 1) >> 1;
+        const int n_items = n_pairs * kSlabs;    // item = (pair, slab), pair-major
+        const int64_t wave_off = (int64_t)(m0 + wm * WTM - band_lo) * g.N + n0 + wn * WTN;
+        auto issue_item = [&](int it, int stage) __attribute__((always_inline)) {
+            // past the end: all lanes re-read 16 bytes of the last item (the load count per item
+            // is fixed for the vmcnt arithmetic; the data is never used)
+            const bool live = it < n_items;
+            const int itc = min(it, n_items - 1);
+            const int qa = 2 * (itc / kSlabs), qb = min(qa + 1, g.n_peers - 1);
+            const int64_t off = wave_off + (int64_t)(itc % kSlabs) * 16 * g.N;
+            const i32x4 rs_a = make_rsrc((const uint16_t*)g.peer.p[qa] + off);
+            const i32x4 rs_b = make_rsrc((const uint16_t*)g.peer.p[qb] + off);
+#pragma unroll
+            for (int r = 0; r < kItemLoads; ++r)
+                lds_dma_b128_stream(r < 4 ? rs_a : rs_b, region + stage * kItemBytes + r * 1024, live ? pvoff[r & 3] : 0u, 0);
+        };
+#pragma unroll
+        for (int it = 0; it < kAhead; ++it) issue_item(it, it);
+#pragma nounroll
+        for (int pr = 0; pr < n_pairs; ++pr) {
+            const bf16x8 xs = (2 * pr + 1 < g.n_peers) ? xsel[0] : xsel[1];
+#pragma unroll
+            for (int i = 0; i < kSlabs; ++i) {
+                // item (pr, i) has landed when at most the three younger items are outstanding; the
+                // stages are private to the wave, so no barrier
+                __builtin_amdgcn_s_waitcnt(vmcnt_imm((kAhead - 1) * kItemLoads));
+                KR_SCHED_FENCE();
+                bf16x8 y[2 * TN];
+#pragma unroll
+                for (int bj = 0; bj < 2 * TN; ++bj) y[bj] = *(lds_frag)(size_t)(pa[bj] + (i % kAhead) * kItemBytes);
+                KR_SCHED_FENCE();   // all eight reads in flight before the first MFMA waits for one
+#pragma unroll
+                for (int bj = 0; bj < 2 * TN; ++bj)
+                    asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(acc16[i][bj]) : "v"(xs), "v"(y[bj]));
+                // every fragment read has returned before the stage is handed back to the DMA
+                __builtin_amdgcn_s_waitcnt(kLgkm0);
+                KR_SCHED_FENCE();
+                issue_item(pr * kSlabs + i + kAhead, i % kAhead);
+                KR_SCHED_FENCE();
+            }
+        }
+        __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));
+        __syncthreads();   // the ring is handed on (k loop or epilogue patches of other waves)
+    };
     // An empty statement that names every accumulator as an AGPR operand, placed between the
     // phases: with the live ranges cut here the register allocator keeps the accumulators
     // where the MFMAs left them instead of moving them to VGPRs and memory for the next phase.
@@ -424,7 +509,10 @@ __device__ __forceinline__ void gemm_dtl_tile(const GemmArgs& g, unsigned char* 
                 for (int j = 0; j < TN; ++j) asm volatile("" : "+a"(acc[i][j]));
         }
     };
-    if (PEERS_FIRST && mfma_peers) peer_phase();
+    if (PEERS_FIRST && mfma_peers) {
+        if constexpr (MI16) peer_phase16();
+        else peer_phase();
+    }
     pin_accumulators();
 
     // ---- prologue: request k-step 0 and the first loads of step 1; wait for step 0 ------------
@@ -615,13 +703,16 @@ __device__ __forceinline__ void gemm_dtl_tile(const GemmArgs& g, unsigned char* 
                                                 part + ((i * TN + j) * 4 + v) * (WM * WN * 64));
         return;
     }
-    if (!PEERS_FIRST && mfma_peers) peer_phase();
+    if (!PEERS_FIRST && mfma_peers) {
+        if constexpr (MI16) peer_phase16();
+        else peer_phase();
+    }
     pin_accumulators();
     // peers and bias that are already in the accumulators are not added again
     if constexpr (MI16) {
         if (full_tile) {
-            gemm_epilogue<BM, WTM, WTN, TM, TN, true, EP_WAVE>(g, g.n_peers, bias_in_acc ? nullptr : g.bias, acc16, smem, m0, n0,
-                                                               wm, wn, lane, wave);
+            gemm_epilogue<BM, WTM, WTN, TM, TN, true, EP_WAVE>(g, mfma_peers ? 0 : g.n_peers, bias_in_acc ? nullptr : g.bias, acc16,
+                                                               smem, m0, n0, wm, wn, lane, wave);
         } else if constexpr (RAGGED) {
             gemm_epilogue<BM, WTM, WTN, TM, TN, false, EP_WAVE>(g, g.n_peers, g.bias, acc16, smem, m0, n0, wm, wn, lane, wave);
         }
@@ -644,11 +735,12 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_dtl_kernel(const GemmArgs g)
     else gemm_dtl_tile<B_NT, false, false, RAGGED>(g, smem);
 }
 
-// The k loop on 16x16x32 blocks (peers, if any, are added in the epilogue).
+// The same on 16x16x32 blocks (k loop and peer phase).
 template <bool B_NT, bool RAGGED>
 __global__ __launch_bounds__(WM* WN * 64) void gemm_dtl16_kernel(const GemmArgs g) {
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
-    gemm_dtl_tile<B_NT, false, false, RAGGED, true>(g, smem);
+    if (g.peers_on_mfma && g.n_peers > 0 && (g.peers_on_mfma == 1 ? ((blockIdx.x >> 3) & 1) : g.peers_on_mfma == 2)) gemm_dtl_tile<B_NT, true, false, RAGGED, true>(g, smem);
+    else gemm_dtl_tile<B_NT, false, false, RAGGED, true>(g, smem);
 }
 
 }  // namespace
@@ -700,7 +792,7 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_dtl_tail_finish_kernel(const
     // rounds once; every other tile of a bf16 result rounds the product to bf16 first and adds the
     // peers and the bias to that.
     const bool tile_in_band = tile_m * BM >= g.band_row0 && tile_m * BM + BM <= g.band_row0 + g.band_rows;
-    const bool peers_exact = !g.mi16 && g.peers_on_mfma && g.n_peers > 0 && tile_in_band;
+    const bool peers_exact = g.peers_on_mfma && g.n_peers > 0 && tile_in_band;
     const bool bias_exact = g.bias != nullptr && tile_in_band && (g.n_peers == 0 || peers_exact);
     auto add_peers = [&]() {
         for (int pq = 0; pq < g.n_peers; ++pq) {

@@ -297,9 +297,9 @@ def test_gemm_noalloc_entry_checks_arguments_first(lib, monkeypatch):
 def test_gemm_plan_reports_the_dispatch(lib, monkeypatch):
     """kr_gemm_plan names the kernel a shape gets, by the rule the launch itself uses."""
     p = _lib.gemm_plan(8192, 8192, 3584, False, 7, 1024, False, True)        # GEMM + reduce-scatter shape
-    assert p["kernel"] == "gemm_dtl16_kernel" and p["tile"] == 256 and p["mfma"] == "16x16x32" and not p["peers_on_mfma"]
+    assert p["kernel"] == "gemm_dtl16_kernel" and p["tile"] == 256 and p["mfma"] == "16x16x32" and p["peers_on_mfma"]
     p = _lib.gemm_plan(4096, 8192, 1024, False, 7, 4096, True, False)        # every tile streams peers
-    assert p["kernel"] == "gemm_dtl_kernel" and p["mfma"] == "32x32x16" and p["peers_on_mfma"] and p["group_n"] == 16
+    assert p["kernel"] == "gemm_dtl16_kernel" and p["mfma"] == "16x16x32" and p["peers_on_mfma"] and p["group_n"] == 16
     p = _lib.gemm_plan(8192, 3584, 8192, True)                               # all-gather matmul shape
     assert p["kernel"] == "gemm_dtl16_kernel" and p["group_n"] == 4 and p["tail_tiles"] == 0
     p = _lib.gemm_plan(256, 256, 100 * 8, False)                             # K not a multiple of 64
