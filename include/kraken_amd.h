@@ -445,6 +445,23 @@ int kr_reduce_rotated_bf16(const void* in, int W, int64_t rows, int64_t N, int r
                            int acc_bf16, void* out, void* stream);
 
 /*
+ * fp32 operands for the bf16 GEMM entry points: x = hi + lo with hi = bf16(x), lo = bf16(x - hi),
+ * written in one pass as the three bf16 blocks of a product that is three times as long:
+ *   [a_hi | a_hi | a_lo] @ [b_hi ; b_lo ; b_hi] = a_hi b_hi + a_hi b_lo + a_lo b_hi
+ * (a @ b without the a_lo b_lo term: about 16 mantissa bits, fp32 accumulate).  The reference
+ * passes fp32 operands to tl.dot, which multiplies them in TF32
+ * (kraken/fused/gemm_one_shot_all_reduce_fused.py:56-64, test/test_gemm_allreduce.py:57-58).
+ *   x: [rows, cols] fp32, row stride ld_x (elements), columns contiguous; cols % 8 == 0
+ *   side_by_side != 0: out is [rows, 3*cols] bf16, block b of a row at columns [b*cols, (b+1)*cols)
+ *                      (row stride ld_out >= 3*cols) -- an operand whose reduction dimension is contiguous
+ *   side_by_side == 0: out is [3*rows, cols] bf16, block b at rows [b*rows, (b+1)*rows)
+ *                      (row stride ld_out >= cols) -- a row-major right operand [K, N]
+ *   pattern 0: blocks hi, hi, lo (left operand); 1: hi, lo, hi (right operand)
+ */
+int kr_split_fp32(const void* x, int64_t rows, int64_t cols, int64_t ld_x, int side_by_side, int pattern,
+                  void* out, int64_t ld_out, void* stream);
+
+/*
  * Which kernel kr_gemm_reduce_*_bf16 would run for a shape (contiguous operands), decided by the
  * same code that launches it; for benchmarks and logs that want to name the kernel they timed.
  * No counterpart in the reference (its tile sizes are keyword arguments of the wrappers,

@@ -108,6 +108,7 @@ _SIGNATURES = {
     "kr_copy_engine_memcpy": (c_int, [c_void_p, c_void_p, c_int64, c_void_p]),
     "kr_flag_arrive_wait": (c_int, [c_void_p, c_int, c_int, c_int64, c_void_p, c_void_p]),
     "kr_reduce_rotated_bf16": (c_int, [c_void_p, c_int, c_int64, c_int64, c_int, c_int, c_void_p, c_void_p]),
+    "kr_split_fp32": (c_int, [c_void_p, c_int64, c_int64, c_int64, c_int, c_int, c_void_p, c_int64, c_void_p]),
     "kr_gemm_plan": (c_int, [c_int64, c_int64, c_int64, c_int, c_int, c_int64, c_int, c_int, c_int64, c_void_p]),
     "kr_probe_read": (c_int, [c_void_p, c_int64, c_void_p, c_void_p]),
     "kr_probe_copy": (c_int, [c_void_p, c_void_p, c_int64, c_void_p]),

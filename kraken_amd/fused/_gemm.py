@@ -15,20 +15,53 @@ def split_fp32(a: torch.Tensor, b: torch.Tensor) -> tuple[torch.Tensor, torch.Te
     length, fp32 accumulate) equals ``a@b`` up to the dropped ``a_lo@b_lo``
     term, i.e. about 16 mantissa bits — tighter than the TF32 ``tl.dot`` the
     reference runs fp32 inputs through (``gemm_one_shot_all_reduce_fused.py:56-64``).
+    Each operand is split in one pass of ``kr_split_fp32`` over it (read fp32 once,
+    write the three bf16 blocks); operands whose layout that kernel does not take
+    (K or N not a multiple of 8, a column-major left operand, rows not 16-byte
+    aligned) are made contiguous first, or, for odd sizes, split by elementwise torch ops.
     """
-    a_hi = a.to(torch.bfloat16)
-    a_lo = (a - a_hi.float()).to(torch.bfloat16)
-    b_hi = b.to(torch.bfloat16)
-    b_lo = (b - b_hi.float()).to(torch.bfloat16)
-    return torch.cat([a_hi, a_hi, a_lo], dim=1), torch.cat([b_hi, b_lo, b_hi], dim=0)
+    M, K = a.shape
+    N = b.shape[1]
+    if not (a.is_cuda and b.is_cuda) or K % 8 != 0 or N % 8 != 0:
+        a_hi = a.to(torch.bfloat16)
+        a_lo = (a - a_hi.float()).to(torch.bfloat16)
+        b_hi = b.to(torch.bfloat16)
+        b_lo = (b - b_hi.float()).to(torch.bfloat16)
+        return torch.cat([a_hi, a_hi, a_lo], dim=1), torch.cat([b_hi, b_lo, b_hi], dim=0)
+    lib = _lib.load()
+    dev = _lib.require_device(a, b)
+    stream = _lib.current_stream(dev)
+
+    def rows_ok(t):      # columns contiguous, rows 16-byte aligned
+        return t.stride(1) == 1 and t.stride(0) % 4 == 0 and t.stride(0) >= t.shape[1] and t.data_ptr() % 16 == 0
+
+    if not rows_ok(a):
+        a = a.contiguous()
+    a3 = torch.empty((M, 3 * K), dtype=torch.bfloat16, device=dev)
+    _lib.check(lib.kr_split_fp32(a.data_ptr(), M, K, a.stride(0), 1, 0, a3.data_ptr(), 3 * K, stream), "split_fp32(a)")
+    if rows_ok(b.T) and not rows_ok(b):
+        # transposed-contiguous right operand: memory is [N, K]; the blocks lie side by side along K
+        bt = b.T
+        b3t = torch.empty((N, 3 * K), dtype=torch.bfloat16, device=dev)
+        _lib.check(lib.kr_split_fp32(bt.data_ptr(), N, K, bt.stride(0), 1, 1, b3t.data_ptr(), 3 * K, stream), "split_fp32(b)")
+        return a3, b3t.T
+    if not rows_ok(b):
+        b = b.contiguous()
+    b3 = torch.empty((3 * K, N), dtype=torch.bfloat16, device=dev)
+    _lib.check(lib.kr_split_fp32(b.data_ptr(), K, N, b.stride(0), 0, 1, b3.data_ptr(), N, stream), "split_fp32(b)")
+    return a3, b3
 
 
 def prepare_operands(a: torch.Tensor, b: torch.Tensor) -> tuple[torch.Tensor, torch.Tensor]:
     """Return bf16 operands in a layout the kernel reads directly.
 
-    A must be k-contiguous; B either row-major or transposed-contiguous.  Other
-    stridings (the reference accepts any 2-D strides) are made contiguous.
-    K and N are padded to multiples of 8 with zeros when necessary.
+    A must be k-contiguous; B either row-major or transposed-contiguous; any row
+    stride that is a multiple of 8 elements is read in place (the kernels address
+    operands through buffer descriptors built from the caller's strides).  Other
+    stridings (the reference accepts any 2-D strides,
+    ``gemm_one_shot_all_reduce_fused.py:163-166``) take one copy.  fp32 operands are
+    split into bf16 parts by one kernel pass each (``split_fp32``).
+    K is padded to a multiple of 8 with zeros when necessary.
     """
     assert a.dim() == 2 and b.dim() == 2
     assert a.shape[1] == b.shape[0], "Inner dimensions must match for matrix multiplication"

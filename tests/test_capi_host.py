@@ -325,6 +325,18 @@ def test_gemm_plan_reports_the_dispatch(lib, monkeypatch):
         _lib.reload_env()
 
 
+def test_split_fp32_argument_errors(lib):
+    f = lib.kr_split_fp32
+    assert f(FAKE, 16, 12, 12, 1, 0, FAKE, 36, None) == _lib.KR_ERR_NUMEL_MOD8
+    assert f(None, 16, 16, 16, 1, 0, FAKE, 48, None) == _lib.KR_ERR_NULL_POINTER
+    assert f(FAKE, 16, 16, 8, 1, 0, FAKE, 48, None) == _lib.KR_ERR_LAYOUT          # row stride shorter than the row
+    assert f(FAKE, 16, 16, 16, 1, 0, FAKE, 40, None) == _lib.KR_ERR_LAYOUT         # side by side needs 3 * cols
+    assert f(FAKE + 4, 16, 16, 16, 1, 0, FAKE, 48, None) == _lib.KR_ERR_ALIGNMENT
+    assert f(FAKE, 16, 16, 18, 1, 0, FAKE, 48, None) == _lib.KR_ERR_ALIGNMENT      # fp32 rows not 16-byte aligned
+    assert f(FAKE, 16, 16, 16, 1, 2, FAKE, 48, None) == _lib.KR_ERR_BAD_DIM
+    assert f(None, 0, 16, 16, 1, 0, None, 48, None) == 0
+
+
 def test_probe_argument_errors(lib):
     assert lib.kr_probe_read(FAKE, 24, None, None) == _lib.KR_ERR_NUMEL_MOD8
     assert lib.kr_probe_read(None, 32, None, None) == _lib.KR_ERR_NULL_POINTER

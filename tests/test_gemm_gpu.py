@@ -65,6 +65,34 @@ def test_gemm_all_reduce_shapes(dev, tile, shape, b_t):
     torch.testing.assert_close(plain.cpu(), orc.gemm_all_reduce(a, b), rtol=1e-3, atol=1e-3)
 
 
+def test_split_fp32_is_one_pass_and_bit_exact(dev):
+    """kr_split_fp32 writes the hi / lo blocks of an fp32 operand in the three layouts the GEMM
+    wrappers use, bit for bit what elementwise torch ops give (hi = bf16(x), lo = bf16(x - hi)),
+    also for a row stride larger than the row."""
+    from kraken_amd.fused import _gemm
+    g = torch.Generator().manual_seed(7)
+    for (M, K, N) in [(64, 128, 72), (300, 264, 136), (8, 8, 8)]:
+        a = torch.randn(M, K + 8, generator=g).to(dev)[:, :K]            # row stride K + 8
+        b = torch.randn(K, N, generator=g).to(dev)
+        bt = torch.randn(N, K, generator=g).to(dev).T                     # transposed-contiguous [K, N]
+        for (x, y) in ((a, b), (a, bt)):
+            a3, b3 = _gemm.split_fp32(x, y)
+            x_hi = x.to(BF16); x_lo = (x - x_hi.float()).to(BF16)
+            y_hi = y.to(BF16); y_lo = (y - y_hi.float()).to(BF16)
+            assert torch.equal(a3, torch.cat([x_hi, x_hi, x_lo], dim=1))
+            assert torch.equal(b3, torch.cat([y_hi, y_lo, y_hi], dim=0))
+            assert b3.T.is_contiguous() == (y is bt)                      # the operand's layout is kept
+            # the 3K-long bf16 product is a @ b to ~16 mantissa bits
+            ref = x.double() @ y.double()
+            got = (a3.double() @ b3.double())
+            assert (got - ref).abs().max() <= 2e-4 * ref.abs().max() + 1e-6
+    # sizes the kernel does not take fall back to elementwise ops with the same result
+    a = torch.randn(16, 12, generator=g).to(dev); b = torch.randn(12, 20, generator=g).to(dev)
+    a3, b3 = _gemm.split_fp32(a, b)
+    assert a3.shape == (16, 36) and b3.shape == (36, 20)
+    assert torch.equal(a3[:, :12], a.to(BF16)) and torch.equal(b3[12:24], (b - b.to(BF16).float()).to(BF16))
+
+
 def test_fp32_operands_reference_shapes(dev, tile):
     # test/test_gemm_allreduce.py:51-89: fp32 N(0,1) operands, (512,256,128) and (256,256,256), tol 1e-1
     for (M, N, K) in [(512, 256, 128), (256, 256, 256)]:
