@@ -66,16 +66,17 @@ MIN_EAGER_STEPS = 30             # timed launches of a side workload that is not
 # profiles/ (one file per kernel and workload).  Each entry: (bytes, commit of the kernel source the
 # profile was taken at); the JSON carries both, so a figure that predates a kernel change shows.
 MEASURED_TRAFFIC = {
-    "one_shot_reduce_w8_4096x4096": (302053204, "69f8a68"),             # profiles/reduce_kernel_w8_4096x4096.md
-    "two_shot_share_w8_512x4096": (37839283, "69f8a68"),                # profiles/reduce_kernel_w8_two_shot_share_512x4096.md
-    "reduce_bias_rmsnorm_w8_256x4096": (19050022, "69f8a68"),           # profiles/reduce_rmsnorm_kernel_w8_256x4096.md
-    "reduce_bias_rmsnorm_w8_16x8192_decode": (2483922, "514d8fc"),      # profiles/reduce_rmsnorm_split_kernel_w8_16x8192.md
-    "reduce_bias_rmsnorm_w8_16384x4096_large": (1208025963, "69f8a68"), # profiles/reduce_rmsnorm_kernel_w8_16384x4096.md
+    "one_shot_reduce_w8_4096x4096": (302051604, "8eb5098"),             # profiles/reduce_kernel_w8_4096x4096.md
+    "two_shot_share_w8_512x4096": (37836204, "8eb5098"),                # profiles/reduce_kernel_w8_two_shot_share_512x4096.md
+    "reduce_bias_rmsnorm_w8_256x4096": (19048668, "8eb5098"),           # profiles/reduce_rmsnorm_kernel_w8_256x4096.md
+    "reduce_bias_rmsnorm_w8_16x8192_decode": (2494411, "8eb5098"),      # profiles/reduce_rmsnorm_split_kernel_w8_16x8192.md
+    "reduce_bias_rmsnorm_w8_16384x4096_large": (1208007579, "8eb5098"), # profiles/reduce_rmsnorm_kernel_w8_16384x4096.md
     # the GEMMs: L2 fills (A and B panels re-read per tile row / column, served mostly by the 256 MB
     # last-level cache, not by HBM) + write-backs
-    "gemm_reduce_scatter_8192x8192x3584_w8": (962243626, "3221dc9"),    # profiles/gemm_dtl16_kernel_reduce_scatter_8192x8192x3584.md
-    "gemm_all_reduce_4096x8192x1024_w8": (705354977, "3221dc9"),        # profiles/gemm_dtl_kernel_all_reduce_4096x8192x1024.md
-    "all_gather_matmul_8192x3584x8192_w8": (875039914, "3221dc9"),      # profiles/gemm_dtl16_kernel_all_gather_matmul_8192x3584x8192.md
+    "gemm_reduce_scatter_8192x8192x3584_w8": (985098980, "8eb5098"),    # profiles/gemm_dtl16_kernel_reduce_scatter_8192x8192x3584.md
+    "gemm_all_reduce_4096x8192x1024_w8": (708000078, "8eb5098"),        # profiles/gemm_dtl16_kernel_all_reduce_4096x8192x1024.md
+    "all_gather_matmul_8192x3584x8192_w8": (876206400, "8eb5098"),      # profiles/gemm_dtl16_kernel_all_gather_matmul_8192x3584x8192.md
+    "all_gather_matmul_4096x6656x16384_w8": (1816571183, "8eb5098"),    # profiles/gemm_dtl16_kernel_all_gather_matmul_4096x6656x16384.md
 }
 
 # Targets of the benchmark definition: fraction of the binding roof.  The W = 8 reduce(+bias+RMSNorm)
