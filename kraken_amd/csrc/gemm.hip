@@ -500,20 +500,6 @@ static int static_scratch(void** out) {
     return KR_OK;
 }
 
-// Compute units of the current device (the persistent kernel's grid), looked up once per device.
-static int compute_units() {
-    static std::atomic<int> cached[kMaxDevices];
-    int dev = 0;
-    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return 256;
-    int n = cached[dev].load(std::memory_order_relaxed);
-    if (n == 0) {
-        if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
-        cached[dev].store(n, std::memory_order_relaxed);
-    }
-    return n;
-}
-static bool kPersistDefault(int env) { return env == 1; }   // off unless asked for
-
 // ---- which kernel a call gets ----------------------------------------------------------------
 // One place decides it, for the launch and for kr_gemm_plan (which reports the decision).
 struct GemmPlan {
@@ -716,16 +702,6 @@ static int gemm_reduce(const void* A, int64_t lda_m, int64_t lda_k, const void* 
     }
     g.peers_on_mfma = plan.peers_on_mfma;
     g.mi16 = plan.mi16;
-    // Persistent form of the 256x256 kernel (one workgroup per compute unit walks the tile order and
-    // requests the next tile's first operands before it stores the current tile): whole tiles of
-    // 16x16 blocks, bf16 result, nothing for the epilogue to load -- peers and bias, if any, are in
-    // the accumulators, which needs bands that begin and end at tile boundaries -- and no flags to
-    // wait for or to set.  KRAKEN_AMD_GEMM_PERSIST=0|1 overrides the default.
-    g.persist = 0;
-    if (dtl && plan.mi16 && M % 256 == 0 && N % 256 == 0 && !out_is_fp32 && g.progress == nullptr &&
-        g.band_counter == nullptr && band_row0 % 256 == 0 && band_rows % 256 == 0 &&
-        (n_peers == 0 || plan.peers_on_mfma != 0) && env_switches().gemm_persist != 0 && kPersistDefault(env_switches().gemm_persist))
-        g.persist = compute_units();
     const int bm = plan.tile, bn = bm;
     g.tiles_m = (int)((M + bm - 1) / bm);
     g.tiles_n = (int)((N + bn - 1) / bn);

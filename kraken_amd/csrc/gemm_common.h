@@ -40,8 +40,7 @@ struct GemmArgs {
     int tail_tiles;
     int group_n;         // column panels per scheduling group (tile_schedule)
     int peers_on_mfma;   // 256x256 kernel: add whole-band tiles' peers through the matrix cores
-    int mi16;            // 256x256 kernel: k loop and peer phase on 16x16x32 MFMA blocks
-    int persist;         // 256x256 kernel: > 0: persistent form with this many workgroups (the GPU's compute units)
+    int mi16;            // 256x256 kernel: k loop on 16x16x32 MFMA blocks (peers in the epilogue)
     // producer of the copy-engine reduce-scatter (band_counter == nullptr: off): finished tiles are
     // counted per destination rank, whose band is count_rows rows of C
     uint32_t* band_counter;   // [M / count_rows] tiles finished that touch the band
@@ -162,13 +161,7 @@ __device__ __forceinline__ void tile_schedule(const GemmArgs& g, int pid, int& t
 // ACC is either f32x16[TM][TN] (32x32 MFMA blocks: lane l holds row l%32 of a block and the
 // columns 8(v/4) + 4(l/32) + v%4 of register v) or f32x4[2*TM][2*TN] (16x16 blocks: lane l
 // holds row l%16 and the columns 4(l/16) + v); only the copy into the patch knows which.
-//
-// SWZ (bf16 result on 16x16 blocks only): the patch has no row padding -- 32 rows of WTN bf16, the
-// 16-byte chunks of a row XOR-swizzled with the row instead -- and lies at `smem` + wave * 32 * WTN * 2
-// bytes: four waves' patches then fit the 32 KiB of LDS that the operand ring leaves free, so the
-// ring can already receive the next tile's operands while this tile is stored (the persistent
-// kernel).
-template <bool F32, int BM, int WTM, int WTN, int TM, int TN, bool EVEN, int EP_WAVE, bool SWZ, class ACC>
+template <bool F32, int BM, int WTM, int WTN, int TM, int TN, bool EVEN, int EP_WAVE, class ACC>
 __device__ __forceinline__ void gemm_epilogue_impl(const GemmArgs& g, const int n_peers, const uint16_t* bias,
                                                    const ACC& acc, unsigned char* smem,
                                                    int m0, int n0, int wm, int wn, int lane, int wave) {
@@ -188,10 +181,9 @@ __device__ __forceinline__ void gemm_epilogue_impl(const GemmArgs& g, const int 
     typedef typename std::conditional<F32, float, uint16_t>::type patch_t;
     // row pitch in elements: 16 bytes of padding keep the quad stores of 16 (bf16: 8-byte) or
     // 8 (fp32: 16-byte) lanes on distinct banks and the rows 16-byte aligned
-    static_assert(!SWZ || (!F32 && MI16 && WTN == 128), "the swizzled patch is written for bf16 results of 16x16 blocks");
-    constexpr int LD = SWZ ? WTN : WTN + (F32 ? 4 : 8);
-    static_assert(SWZ || 32 * LD * (int)sizeof(patch_t) <= EP_WAVE, "patch exceeds the wave's share of LDS");
-    patch_t* patch = (patch_t*)(smem + wave * (SWZ ? 32 * WTN * 2 : EP_WAVE));
+    constexpr int LD = WTN + (F32 ? 4 : 8);
+    static_assert(32 * LD * (int)sizeof(patch_t) <= EP_WAVE, "patch exceeds the wave's share of LDS");
+    patch_t* patch = (patch_t*)(smem + wave * EP_WAVE);
     constexpr int CPR = WTN / 8;            // 8-element chunks per patch row
     constexpr int EP_ITERS = 32 * CPR / 64; // chunks per lane per 32-row slab
     constexpr int kChunkBatch = BM >= 256 ? 4 : 2;   // the small tile keeps its register count low (occupancy)
@@ -239,14 +231,7 @@ __device__ __forceinline__ void gemm_epilogue_impl(const GemmArgs& g, const int 
                                 *(f32x4*)(row + h * 16 * LD + j * 16) = a;
                             } else {
                                 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
-                                if constexpr (SWZ) {
-                                    // row lane%16 + 16h, columns 16j + 4(lane/16) .. +3: chunk 2j + (lane/32), half (lane/16)%2
-                                    patch_t* dst = patch + ((lane & 15) + 16 * h) * LD +
-                                                   (((2 * j + (lane >> 5)) ^ (lane & 15)) << 3) + 4 * ((lane >> 4) & 1);
-                                    *(u32x2*)dst = u32x2{pack_here(a[0], a[1]), pack_here(a[2], a[3])};
-                                } else {
-                                    *(u32x2*)(row + h * 16 * LD + j * 16) = u32x2{pack_here(a[0], a[1]), pack_here(a[2], a[3])};
-                                }
+                                *(u32x2*)(row + h * 16 * LD + j * 16) = u32x2{pack_here(a[0], a[1]), pack_here(a[2], a[3])};
                             }
                         }
                 } else {
@@ -276,8 +261,7 @@ __device__ __forceinline__ void gemm_epilogue_impl(const GemmArgs& g, const int 
     // one chunk of the current slab: as stored (bf16 patch) or as fp32 values
     auto read_raw = [&](int chunk) __attribute__((always_inline)) {
         const int r = chunk * (64 / CPR) + lane_r;
-        if constexpr (SWZ) return *(const u32x4*)(patch + r * LD + ((lane_cc ^ (r & 15)) << 3));
-        else return *(const u32x4*)(patch + r * LD + lane_cc * 8);
+        return *(const u32x4*)(patch + r * LD + lane_cc * 8);
     };
     auto read_chunk = [&](int chunk, float (&f)[8]) __attribute__((always_inline)) {
         if constexpr (F32) {
@@ -481,18 +465,9 @@ template <int BM, int WTM, int WTN, int TM, int TN, bool EVEN, int EP_WAVE, clas
 __device__ __forceinline__ void gemm_epilogue(const GemmArgs& g, int n_peers, const uint16_t* bias,
                                               const ACC& acc, unsigned char* smem,
                                               int m0, int n0, int wm, int wn, int lane, int wave) {
-    if (g.out_is_fp32) gemm_epilogue_impl<true, BM, WTM, WTN, TM, TN, EVEN, EP_WAVE, false, ACC>(g, n_peers, bias, acc, smem, m0, n0, wm, wn, lane, wave);
-    else gemm_epilogue_impl<false, BM, WTM, WTN, TM, TN, EVEN, EP_WAVE, false, ACC>(g, n_peers, bias, acc, smem, m0, n0, wm, wn, lane, wave);
+    if (g.out_is_fp32) gemm_epilogue_impl<true, BM, WTM, WTN, TM, TN, EVEN, EP_WAVE, ACC>(g, n_peers, bias, acc, smem, m0, n0, wm, wn, lane, wave);
+    else gemm_epilogue_impl<false, BM, WTM, WTN, TM, TN, EVEN, EP_WAVE, ACC>(g, n_peers, bias, acc, smem, m0, n0, wm, wn, lane, wave);
     if (g.band_counter != nullptr) count_finished_tile(g, m0, BM);
-}
-
-// The bf16 epilogue of a whole tile whose rows lie all inside or all outside the band and that
-// has nothing left to add (no peers, no bias), out of the swizzled patch at `spare` (LDS outside
-// the operand ring): conversions, LDS round trip and stores only, no loads.
-template <int BM, int WTM, int WTN, int TM, int TN, class ACC>
-__device__ __forceinline__ void gemm_epilogue_plain_bf16(const GemmArgs& g, const ACC& acc, unsigned char* spare,
-                                                         int m0, int n0, int wm, int wn, int lane, int wave) {
-    gemm_epilogue_impl<false, BM, WTM, WTN, TM, TN, true, 0, true, ACC>(g, 0, nullptr, acc, spare, m0, n0, wm, wn, lane, wave);
 }
 
 }  // namespace kr

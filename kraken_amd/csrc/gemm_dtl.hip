@@ -29,8 +29,6 @@
 // hold C transposed: a lane owns one row m and four consecutive columns n per register quad,
 // which is what the fused epilogue (gemm_common.h) stores and what lets the partial sums of the
 // other ranks be added by the matrix cores themselves (peer_phase below).
-#include <algorithm>
-
 #include "gemm_common.h"
 
 namespace kr {
@@ -48,8 +46,6 @@ constexpr int LDS_BYTES = NSTAGE * (A_ST + B_ST);
 constexpr int LOADS_A = A_ST / 1024 / (WM * WN);   // LDS-DMA loads (1 KiB each) per wave per k-step: 8 A ...
 constexpr int LOADS_PER_TILE = 2 * LOADS_A;        // ... + 8 B
 constexpr int EP_WAVE = 32 * (WTN + 4) * 4;     // epilogue patch of a wave: 32 rows x WTN fp32, padded
-constexpr int kEpilogueStores = WTM * WTN * 2 / 1024;   // 16-byte stores per lane of a wave's bf16 tile part (32)
-constexpr int LDS_BYTES_PERSIST = 160 * 1024;   // the ring + four swizzled bf16 patches of 8 KiB
 static_assert(EP_WAVE * WM * WN <= LDS_BYTES, "epilogue patch must fit in the operand ring");
 
 typedef __attribute__((address_space(3))) void* lds_void;
@@ -70,16 +66,8 @@ constexpr int kLgkm0 = 0xc07f;   // s_waitcnt lgkmcnt(0) only
 // 32x32x16 (4 x 4 blocks of 32 x 32): same operand traffic, but the matrix cores draw less power
 // per flop with it (under the power limit, matrix-core-only loops on random operands sustain
 // 2.04 PFLOP/s with 16x16x32 against 1.62 with 32x32x16).
-// PERSIST: the workgroup runs the tiles  blockIdx.x, blockIdx.x + gridDim.x, ...  of the order, one
-// after the other, and requests the first operands of the next tile BEFORE it stores the current
-// one: the loads travel while the epilogue runs, and the stores drain while the next k loop runs
-// (a workgroup that ends after every tile waits for its stores, and its successor for its first
-// loads).  For that the epilogue works out of the 32 KiB of LDS beside the operand ring.  Only
-// for whole tiles of 16x16 blocks with a bf16 result whose epilogue has nothing to load (peers and
-// bias, if any, already in the accumulators; bands that begin and end at tile boundaries).
-template <bool B_NT, bool PEERS_FIRST, bool SPLIT = false, bool RAGGED = false, bool MI16 = false, bool PERSIST = false>
+template <bool B_NT, bool PEERS_FIRST, bool SPLIT = false, bool RAGGED = false, bool MI16 = false>
 __device__ __forceinline__ void gemm_dtl_tile(const GemmArgs& g, unsigned char* smem) {
-    static_assert(!PERSIST || (MI16 && !SPLIT && !RAGGED), "persistent form: 16x16 blocks, whole tiles, no split");
     // Nothing is outstanding at kernel entry; saying so keeps the compiler's own wait-count
     // bookkeeping from carrying the pending loads and stores of the other copy of this code
     // (which never runs in the same workgroup) into this one, where it cannot see the LDS-DMA
@@ -94,10 +82,9 @@ __device__ __forceinline__ void gemm_dtl_tile(const GemmArgs& g, unsigned char* 
     const int first_tile = g.tiles_m * g.tiles_n - g.tail_tiles;     // SPLIT: tiles the main launch took
     const int split = SPLIT ? (int)(blockIdx.x % (unsigned)g.k_splits) : 0;
     const int tail_index = SPLIT ? (int)(blockIdx.x / (unsigned)g.k_splits) : 0;
-    int wg_virtual = blockIdx.x;                                     // PERSIST: advances by gridDim.x per tile
-    tile_schedule(g, SPLIT ? schedule_position(g, tail_index, first_tile) : schedule_position(g, wg_virtual), tile_m,
+    tile_schedule(g, SPLIT ? schedule_position(g, tail_index, first_tile) : schedule_position(g, blockIdx.x), tile_m,
                   tile_n);
-    int m0 = tile_m * BM, n0 = tile_n * BN;
+    const int m0 = tile_m * BM, n0 = tile_n * BN;
     // k-steps of this workgroup: all of them, or the split's share
     const int kt_all = g.K / BKD;
     const int kt_begin = SPLIT ? (int)((int64_t)kt_all * split / g.k_splits) : 0;
@@ -162,8 +149,8 @@ __device__ __forceinline__ void gemm_dtl_tile(const GemmArgs& g, unsigned char* 
                      : "s"(lds_addr), "v"(voff), "s"(rsrc), "s"(soff)
                      : "memory", "m0");
     };
-    i32x4 a_rsrc = RAGGED ? make_rsrc(a_tile, ((int64_t)(rows_a - 1) * lda + (g.K - k_begin)) * 2) : make_rsrc(a_tile);
-    i32x4 bt_rsrc = RAGGED ? make_rsrc(g.B + (int64_t)n0 * g.ldb + (B_NT ? k_begin : 0),
+    const i32x4 a_rsrc = RAGGED ? make_rsrc(a_tile, ((int64_t)(rows_a - 1) * lda + (g.K - k_begin)) * 2) : make_rsrc(a_tile);
+    const i32x4 bt_rsrc = RAGGED ? make_rsrc(g.B + (int64_t)n0 * g.ldb + (B_NT ? k_begin : 0),
                                              ((int64_t)(rows_b - 1) * g.ldb + (g.K - k_begin)) * 2)
                                  : make_rsrc(g.B + (int64_t)n0 * g.ldb + (B_NT ? k_begin : 0));
 
@@ -285,9 +272,9 @@ __device__ __forceinline__ void gemm_dtl_tile(const GemmArgs& g, unsigned char* 
     // values, the same for all four row blocks.
     const int band_lo = g.band_row0;
     const bool full_tile = !RAGGED || (m0 + BM <= g.M && n0 + BN <= g.N);
-    bool tile_in_band = full_tile && m0 >= band_lo && m0 + BM <= band_lo + g.band_rows;
-    bool mfma_peers = !SPLIT && g.peers_on_mfma && g.n_peers > 0 && tile_in_band;
-    bool bias_in_acc = !SPLIT && g.bias != nullptr && tile_in_band && (g.n_peers == 0 || mfma_peers);
+    const bool tile_in_band = full_tile && m0 >= band_lo && m0 + BM <= band_lo + g.band_rows;
+    const bool mfma_peers = !SPLIT && g.peers_on_mfma && g.n_peers > 0 && tile_in_band;
+    const bool bias_in_acc = !SPLIT && g.bias != nullptr && tile_in_band && (g.n_peers == 0 || mfma_peers);
     f32x16 acc[TM][TN];
     {
         f32x16 init[TN];
@@ -317,8 +304,8 @@ __device__ __forceinline__ void gemm_dtl_tile(const GemmArgs& g, unsigned char* 
 
     // the same for the 16x16 blocks: a lane holds row lane%16 and the columns 16j + 4(lane/16) .. +3
     f32x4 acc16[2 * TM][2 * TN];
-    f32x4 init16[2 * TN];      // initial value of a row of blocks: zero, or the bias of the tile's columns
-    auto load_init16 = [&]() __attribute__((always_inline)) {
+    if constexpr (MI16) {
+        f32x4 init16[2 * TN];
 #pragma unroll
         for (int j = 0; j < 2 * TN; ++j) init16[j] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
         if (bias_in_acc) {
@@ -330,13 +317,11 @@ __device__ __forceinline__ void gemm_dtl_tile(const GemmArgs& g, unsigned char* 
                 init16[j] = f32x4{bf16_lo(b4.x), bf16_hi(b4.x), bf16_lo(b4.y), bf16_hi(b4.y)};
             }
         }
-    };
-    if constexpr (MI16) load_init16();
-    // PERSIST: what of the next tile has been requested before the previous tile's stores (0: nothing,
-    // 1: stage 0 of its k loop, 2: the first items of its peer phase), and how many stores lie
-    // between those requests and whatever this tile issues next -- stores and loads retire through
-    // one in-order counter, so a wait for the early requests must allow for the younger stores.
-    int pre_kind = 0, pre_stores = 0;
+#pragma unroll
+        for (int i = 0; i < 2 * TM; ++i)
+#pragma unroll
+            for (int j = 0; j < 2 * TN; ++j) acc16[i][j] = init16[j];
+    }
 
 #define KR_SCHED_FENCE() __builtin_amdgcn_sched_barrier(0)
     // ---- partial sums of the other ranks, added on the matrix cores ---------------------------
@@ -430,7 +415,7 @@ __device__ __forceinline__ void gemm_dtl_tile(const GemmArgs& g, unsigned char* 
     // a, rows 16..31: peer b; 8 KiB, eight LDS-DMA loads); half as many MFMA cycles per peer as the
     // 32x32x16 form.  An odd peer count repeats the last peer as b and masks it in X (a product
     // 0 * finite adds nothing).
-    auto peer_phase16 = [&](bool only_issue = false) __attribute__((always_inline)) {
+    auto peer_phase16 = [&]() __attribute__((always_inline)) {
         constexpr int kItemLoads = 8;
         constexpr int kItemBytes = kItemLoads * 1024;
         constexpr int kAhead = 4;
@@ -480,13 +465,8 @@ __device__ __forceinline__ void gemm_dtl_tile(const GemmArgs& g, unsigned char* 
             for (int r = 0; r < kItemLoads; ++r)
                 lds_dma_b128_stream(r < 4 ? rs_a : rs_b, region + stage * kItemBytes + r * 1024, live ? pvoff[r & 3] : 0u, 0);
         };
-        if (only_issue || pre_kind != 2) {
 #pragma unroll
-            for (int it = 0; it < kAhead; ++it) issue_item(it, it);
-        }
-        if (only_issue) return;
-        // (items requested before the previous tile's stores: those stores are younger than the items)
-        const bool stores_behind = PERSIST && pre_kind == 2 && pre_stores > 0;
+        for (int it = 0; it < kAhead; ++it) issue_item(it, it);
 #pragma nounroll
         for (int pr = 0; pr < n_pairs; ++pr) {
             const bf16x8 xs = (2 * pr + 1 < g.n_peers) ? xsel[0] : xsel[1];
@@ -494,12 +474,7 @@ __device__ __forceinline__ void gemm_dtl_tile(const GemmArgs& g, unsigned char* 
             for (int i = 0; i < kSlabs; ++i) {
                 // item (pr, i) has landed when at most the three younger items are outstanding; the
                 // stages are private to the wave, so no barrier
-                if (PERSIST && i < kAhead && stores_behind && pr == 0) {
-                    static_assert((kAhead - 1) * kItemLoads + kEpilogueStores <= 63, "vmcnt holds six bits");
-                    __builtin_amdgcn_s_waitcnt(vmcnt_imm((kAhead - 1) * kItemLoads + kEpilogueStores));
-                } else {
-                    __builtin_amdgcn_s_waitcnt(vmcnt_imm((kAhead - 1) * kItemLoads));
-                }
+                __builtin_amdgcn_s_waitcnt(vmcnt_imm((kAhead - 1) * kItemLoads));
                 KR_SCHED_FENCE();
                 bf16x8 y[2 * TN];
 #pragma unroll
@@ -534,13 +509,6 @@ __device__ __forceinline__ void gemm_dtl_tile(const GemmArgs& g, unsigned char* 
                 for (int j = 0; j < TN; ++j) asm volatile("" : "+a"(acc[i][j]));
         }
     };
-    for (;;) {   // one trip per tile (a single trip unless PERSIST)
-    if constexpr (MI16) {
-#pragma unroll
-        for (int i = 0; i < 2 * TM; ++i)
-#pragma unroll
-            for (int j = 0; j < 2 * TN; ++j) acc16[i][j] = init16[j];
-    }
     if (PEERS_FIRST && mfma_peers) {
         if constexpr (MI16) peer_phase16();
         else peer_phase();
@@ -559,19 +527,11 @@ __device__ __forceinline__ void gemm_dtl_tile(const GemmArgs& g, unsigned char* 
     // of step t+1)
     constexpr int kEarly = MI16 ? 14 : 6;
     static_assert(NSTAGE == 2 && LOADS_PER_TILE == 16, "load schedule below: 6 + 8 + 2 loads");
-    const bool stage0_requested = PERSIST && pre_kind == 1;
-    if (!stage0_requested) {
 #pragma unroll
-        for (int q = 0; q < LOADS_PER_TILE; ++q) issue_load(0, 0, q);
-    }
+    for (int q = 0; q < LOADS_PER_TILE; ++q) issue_load(0, 0, q);
 #pragma unroll
     for (int q = 0; q < kEarly; ++q) issue_load(1, 1, q);
-    if (PERSIST && stage0_requested && pre_stores > 0) {
-        static_assert(!PERSIST || kEarly + kEpilogueStores <= 63, "vmcnt holds six bits");
-        __builtin_amdgcn_s_waitcnt(vmcnt_imm(PERSIST ? kEarly + kEpilogueStores : 0));
-    } else {
-        __builtin_amdgcn_s_waitcnt(vmcnt_imm(kEarly));
-    }
+    __builtin_amdgcn_s_waitcnt(vmcnt_imm(kEarly));
     __builtin_amdgcn_s_barrier();
     KR_SCHED_FENCE();
     if constexpr (MI16) {   // (A blocks 4..7 are read inside the first sub-step)
@@ -748,41 +708,6 @@ __device__ __forceinline__ void gemm_dtl_tile(const GemmArgs& g, unsigned char* 
         else peer_phase();
     }
     pin_accumulators();
-    if constexpr (PERSIST) {
-        // Every wave has passed the barrier behind its last read of the ring: the ring is free.  Move
-        // on to the next tile of this workgroup -- descriptors, flags, the bias its accumulators
-        // start from, and the first loads of its first phase -- and only then store the current one
-        // (from the patches beside the ring).
-        const int m0_done = m0, n0_done = n0;
-        const bool stored = tile_in_band || g.c_full != nullptr;
-        wg_virtual += (int)gridDim.x;
-        const bool more = wg_virtual < g.tiles_m * g.tiles_n - g.tail_tiles;
-        pre_kind = 0;
-        if (more) {
-            tile_schedule(g, schedule_position(g, wg_virtual), tile_m, tile_n);
-            m0 = tile_m * BM;
-            n0 = tile_n * BN;
-            a_tile = g.A + (int64_t)m0 * g.lda;
-            a_rsrc = make_rsrc(a_tile);
-            bt_rsrc = make_rsrc(g.B + (int64_t)n0 * g.ldb);
-            tile_in_band = m0 >= band_lo && m0 + BM <= band_lo + g.band_rows;
-            mfma_peers = g.peers_on_mfma && g.n_peers > 0 && tile_in_band;
-            bias_in_acc = g.bias != nullptr && tile_in_band && (g.n_peers == 0 || mfma_peers);
-            load_init16();
-            if (PEERS_FIRST && mfma_peers) {
-                peer_phase16(true);
-                pre_kind = 2;
-            } else {
-#pragma unroll
-                for (int q = 0; q < LOADS_PER_TILE; ++q) issue_load(0, 0, q);
-                pre_kind = 1;
-            }
-            pre_stores = stored ? kEpilogueStores : 0;
-        }
-        if (stored) gemm_epilogue_plain_bf16<BM, WTM, WTN, TM, TN>(g, acc16, smem + LDS_BYTES, m0_done, n0_done, wm, wn, lane, wave);
-        if (!more) break;
-        continue;
-    }
     // peers and bias that are already in the accumulators are not added again
     if constexpr (MI16) {
         if (full_tile) {
@@ -797,8 +722,6 @@ __device__ __forceinline__ void gemm_dtl_tile(const GemmArgs& g, unsigned char* 
     } else if constexpr (RAGGED) {   // edge tile: every access checked against M and N
         gemm_epilogue<BM, WTM, WTN, TM, TN, false, EP_WAVE>(g, g.n_peers, g.bias, acc, smem, m0, n0, wm, wn, lane, wave);
     }
-    break;
-    }   // tile loop
 }
 #undef KR_SCHED_FENCE
 
@@ -818,15 +741,6 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_dtl16_kernel(const GemmArgs 
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     if (g.peers_on_mfma && g.n_peers > 0 && (g.peers_on_mfma == 1 ? ((blockIdx.x >> 3) & 1) : g.peers_on_mfma == 2)) gemm_dtl_tile<B_NT, true, false, RAGGED, true>(g, smem);
     else gemm_dtl_tile<B_NT, false, false, RAGGED, true>(g, smem);
-}
-
-// The persistent form of the same: as many workgroups as the GPU has compute units (at most one per
-// tile), each walking the tile order with that stride.
-template <bool B_NT>
-__global__ __launch_bounds__(WM* WN * 64) void gemm_dtl16p_kernel(const GemmArgs g) {
-    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
-    if (g.peers_on_mfma && g.n_peers > 0 && (g.peers_on_mfma == 1 ? ((blockIdx.x >> 3) & 1) : g.peers_on_mfma == 2)) gemm_dtl_tile<B_NT, true, false, false, true, true>(g, smem);
-    else gemm_dtl_tile<B_NT, false, false, false, true, true>(g, smem);
 }
 
 }  // namespace
@@ -920,13 +834,6 @@ hipError_t launch_gemm_dtl(const GemmArgs& g, bool b_nt, hipStream_t st, void* w
         return e;
     if (grid.x == 0) {
         // every tile belongs to the split partial round
-    } else if (g.persist) {
-        static std::atomic<uint64_t> popted[2];
-        const void* pfn = b_nt ? (const void*)gemm_dtl16p_kernel<true> : (const void*)gemm_dtl16p_kernel<false>;
-        if (hipError_t e = lds_opt_in(pfn, LDS_BYTES_PERSIST, popted[b_nt ? 1 : 0]); e != hipSuccess) return e;
-        const dim3 pgrid(std::min<unsigned>(grid.x, (unsigned)g.persist));
-        if (b_nt) hipLaunchKernelGGL((gemm_dtl16p_kernel<true>), pgrid, block, LDS_BYTES_PERSIST, st, g);
-        else hipLaunchKernelGGL((gemm_dtl16p_kernel<false>), pgrid, block, LDS_BYTES_PERSIST, st, g);
     } else if (g.mi16) {
         if (b_nt) {
             if (ragged) hipLaunchKernelGGL((gemm_dtl16_kernel<true, true>), grid, block, LDS_BYTES, st, g);

@@ -21,7 +21,6 @@ static EnvSwitches read_env() {
     e.gemm_group = num("KRAKEN_AMD_GEMM_GROUP");
     e.gemm_splitk = num("KRAKEN_AMD_GEMM_SPLITK");
     e.gemm_tailsplit = num("KRAKEN_AMD_GEMM_TAILSPLIT");
-    e.gemm_persist = num("KRAKEN_AMD_GEMM_PERSIST");
     return e;
 }
 static EnvSwitches& env_storage() {
