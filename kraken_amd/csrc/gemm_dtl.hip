@@ -754,7 +754,9 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_dtl_split_kernel(const GemmA
 }
 
 // Third launch: sums the parts of every tail tile in the order 0..S-1 and applies the epilogue
-// of the one-pass kernel to it (own product in fp32 + peers 0, 1, ... + bias, one rounding).
+// of the one-pass kernel to it, with that kernel's rounding (spelled out at `tile_in_band` below:
+// whole-band tiles sum product, peers and bias in fp32 and round once, every other tile of a bf16
+// result rounds the product first).
 // One thread per accumulator quad: block b = (tail tile, quad q), thread tid as in the GEMM
 // kernel; the quad is row wm*128 + 32i + lane%32, columns wn*128 + 32j + 8(v/4) + 4(lane/32) .. +3.
 __global__ __launch_bounds__(WM* WN * 64) void gemm_dtl_tail_finish_kernel(const GemmArgs g, const f32x4* __restrict__ parts) {
