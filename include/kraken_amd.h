@@ -462,6 +462,22 @@ int kr_split_fp32(const void* x, int64_t rows, int64_t cols, int64_t ld_x, int s
                   void* out, int64_t ld_out, void* stream);
 
 /*
+ * fp8 operands (e4m3fn: bias 7, no infinities, largest finite 448) for the bf16 GEMM entry points,
+ * and fp32 results back to fp8, for the fp8 branch of the all-gather matmul
+ * (kraken/fused/all_gather_matmul.py:53,121,213: fp8 operands, fp32 accumulate, fp8 result).  Every
+ * e4m3 value is a bf16 value, so the bf16 product of converted operands, accumulated in fp32, is
+ * what an fp8 matrix-core instruction with fp32 accumulation computes; the fp32 result is rounded
+ * to fp8 once.
+ *   kr_cast_fp8_to_bf16: dst[i] = bf16(src[i]), exact; src n bytes, dst n bf16.
+ *   kr_cast_f32_to_fp8:  dst[i] = e4m3(src[i]), round to nearest even; finite values of magnitude
+ *     448 and more (infinities included) give +-448 (the saturating conversion the reference's
+ *     generated code uses); NaN stays NaN.
+ * n % 16 == 0; pointers 16-byte aligned; n == 0: nothing is launched.
+ */
+int kr_cast_fp8_to_bf16(const void* src, int64_t n, void* dst, void* stream);
+int kr_cast_f32_to_fp8(const void* src, int64_t n, void* dst, void* stream);
+
+/*
  * Which kernel kr_gemm_reduce_*_bf16 would run for a shape (contiguous operands), decided by the
  * same code that launches it; for benchmarks and logs that want to name the kernel they timed.
  * No counterpart in the reference (its tile sizes are keyword arguments of the wrappers,

@@ -26,10 +26,10 @@ class PeerBuffers:
     Both forms give bit-identical results: the kernels are the same.
     """
 
-    def __init__(self, buffers: torch.Tensor | Sequence[torch.Tensor]):
+    def __init__(self, buffers: torch.Tensor | Sequence[torch.Tensor], dtypes=(torch.bfloat16,)):
         if isinstance(buffers, torch.Tensor):
             assert buffers.dim() >= 2, "expected a stacked tensor of shape [W, ...]"
-            assert buffers.dtype == torch.bfloat16, "Only bfloat16 is supported for now."
+            assert buffers.dtype in dtypes, "Only bfloat16 is supported for now."
             self.W = buffers.shape[0]
             assert self.W >= 1
             assert buffers[0].is_contiguous(), "each of the W slices must be contiguous"
@@ -42,7 +42,7 @@ class PeerBuffers:
             assert len(bufs) >= 1, "expected W >= 1 buffers"
             for t in bufs:
                 assert isinstance(t, torch.Tensor), "expected a tensor or a sequence of tensors"
-                assert t.dtype == torch.bfloat16, "Only bfloat16 is supported for now."
+                assert t.dtype in dtypes and t.dtype == bufs[0].dtype, "Only bfloat16 is supported for now."
                 assert t.is_contiguous(), "each of the W buffers must be contiguous"
                 assert t.shape == bufs[0].shape, "the W buffers must have one shape"
             self.W = len(bufs)

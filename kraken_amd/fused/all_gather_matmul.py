@@ -38,6 +38,44 @@ def _matmul_w_progress(a, a_local, b, progress, configs, status=None) -> torch.T
     return c
 
 
+def _all_gather_matmul_fp8(peers: PeerBuffers, b, a_out, progress, **kwargs):
+    """The fp8 branch of ``all_gather_matmul``: convert, multiply in bf16 with an fp32 result, round once."""
+    fp8 = torch.float8_e4m3fn
+    W = peers.W
+    m, K = peers.slice(0).shape
+    assert b.dtype == fp8, "fp8 shards need an fp8 b"
+    assert b.dim() == 2 and b.shape[0] == K
+    if not b.T.is_contiguous():
+        raise ValueError("b.T must be contiguous")
+    stacked = peers.stacked is not None and peers.stacked.is_contiguous()
+    if kwargs.get("gather", not stacked) or not stacked:
+        raise NotImplementedError("fp8 shards: only the gathered form (one contiguous [W, m, K] tensor, gather=False)")
+    M, N = W * m, b.shape[1]
+    assert K % 16 == 0 and N % 16 == 0 and (M * N) % 16 == 0, "fp8 operands: sizes must be multiples of 16"
+    rank = kwargs.get("rank", 0)
+    assert 0 <= rank < W
+    dev = _lib.require_device(peers.stacked, b, a_out, progress)
+    lib = _lib.load()
+    stream = _lib.current_stream(dev)
+    a_full = peers.stacked.reshape(M, K)
+    if a_out is not None:
+        assert a_out.shape == a_full.shape and a_out.dtype == fp8
+        a_out.copy_(a_full)
+    else:
+        a_out = a_full
+    if progress is not None:
+        progress.fill_(1)
+    a16 = torch.empty((M, K), dtype=torch.bfloat16, device=dev)
+    bt16 = torch.empty((N, K), dtype=torch.bfloat16, device=dev)           # b.T is contiguous: memory [N, K]
+    _lib.check(lib.kr_cast_fp8_to_bf16(a_full.data_ptr(), M * K, a16.data_ptr(), stream), "cast_fp8_to_bf16(a)")
+    _lib.check(lib.kr_cast_fp8_to_bf16(b.T.data_ptr(), N * K, bt16.data_ptr(), stream), "cast_fp8_to_bf16(b)")
+    c32 = torch.empty((M, N), dtype=torch.float32, device=dev)
+    _gemm.launch("all_gather_matmul", a16, bt16.T, M, N, None, 0, 0, None, 0, M, None, c32, rank * m)
+    c = torch.empty((M, N), dtype=fp8, device=dev)
+    _lib.check(lib.kr_cast_f32_to_fp8(c32.data_ptr(), M * N, c.data_ptr(), stream), "cast_f32_to_fp8(c)")
+    return a_out, c
+
+
 def all_gather_matmul(
     a_shared,
     b: torch.Tensor,
@@ -75,8 +113,19 @@ def all_gather_matmul(
     ``rank`` (kwarg, default 0) is consumed first and the others in the order
     the copies are issued (``:93``).  ``splits_per_rank`` (default 1) chunks per
     shard; the remaining tile-size kwargs are accepted and ignored.
+
+    fp8 operands (``torch.float8_e4m3fn`` for the shards and ``b``) give an fp8 ``c``
+    like in the reference (``:53,121,213``): fp32 accumulate, one rounding to fp8
+    (nearest even, magnitudes of 448 and more saturate to 448).  Here the operands
+    are widened to bf16 by one conversion pass each (exact: every e4m3 value is a
+    bf16 value), the bf16 kernels run with an fp32 result, and a third pass rounds
+    that to fp8; ``a_gathered`` stays fp8.  Only for ``gather=False`` and sizes that
+    are multiples of 16.
     """
-    peers = PeerBuffers(a_shared)
+    fp8 = torch.float8_e4m3fn
+    peers = PeerBuffers(a_shared, dtypes=(torch.bfloat16, fp8))
+    if peers.slice(0).dtype == fp8:
+        return _all_gather_matmul_fp8(peers, b, a_out, progress, **kwargs)
     W = peers.W
     shard = peers.slice(0)
     assert shard.dim() == 2, "expected shards of shape [m, K]"

@@ -21,6 +21,13 @@ the reference lines it follows.  What pins each function (see
 * GEMM (+reduce / +band): the closed-form known-answer tests of the reference
   (``test/test_gemm_allreduce.py:92-117``, ``test/test_gemm_reduce_scatter.py:76-91``),
   identity-B, ones x ones = K, and a brute-force triple loop in C.
+* fp8 branch of the all-gather matmul (``all_gather_matmul_fp8``): closed forms on
+  exactly representable values, and a brute-force search of the nearest e4m3 value
+  (ties to the even code) over the table of all 254 finite codes for products
+  computed exactly in float64.  The reference holds no test of this branch and the
+  saturating conversion is read off the instruction Triton emits for
+  ``.to(tl.float8e4nv)`` on NVIDIA hardware: beyond its definition this function is
+  "parity unpinned".
 
 Beyond the tolerance bands of the reference's tests (1e-2 .. 1e-1) the
 reference's bit-level behaviour (Triton ``tl.sum`` tree order, ``rsqrt.approx``,
@@ -199,6 +206,17 @@ def all_gather_matmul(a_stack: torch.Tensor, b: torch.Tensor) -> tuple[torch.Ten
 # --------------------------------------------------------------------------------------
 # Deterministic synthetic inputs of the benchmark configurations
 # --------------------------------------------------------------------------------------
+def all_gather_matmul_fp8(a_stack: torch.Tensor, b: torch.Tensor) -> tuple[torch.Tensor, torch.Tensor]:
+    """The fp8 branch of the all-gather matmul (kraken/fused/all_gather_matmul.py:53,121,213): fp8
+    (e4m3fn) operands, fp32 accumulate, the result rounded to fp8 once.  The rounding is torch's
+    (nearest even), clamped to +-448 first: the reference's generated conversion saturates where
+    torch's gives NaN, from magnitude 464 on."""
+    W, m, K = a_stack.shape
+    a_full = a_stack.reshape(W * m, K)
+    c = torch.matmul(a_full.float(), b.float()).clamp(-448.0, 448.0)
+    return a_full, c.to(torch.float8_e4m3fn)
+
+
 def randn_bf16(shape, seed: int, std: float = 1.0, mean: float = 0.0) -> torch.Tensor:
     """fp32 normal draw from a seeded CPU generator, scaled, cast to bf16."""
     g = torch.Generator(device="cpu")

@@ -337,6 +337,16 @@ def test_split_fp32_argument_errors(lib):
     assert f(None, 0, 16, 16, 1, 0, None, 48, None) == 0
 
 
+def test_fp8_cast_argument_errors(lib):
+    for f in (lib.kr_cast_fp8_to_bf16, lib.kr_cast_f32_to_fp8):
+        assert f(FAKE, 24, FAKE, None) == _lib.KR_ERR_NUMEL_MOD8
+        assert f(FAKE, -16, FAKE, None) == _lib.KR_ERR_BAD_DIM
+        assert f(None, 32, FAKE, None) == _lib.KR_ERR_NULL_POINTER
+        assert f(FAKE, 32, None, None) == _lib.KR_ERR_NULL_POINTER
+        assert f(FAKE + 4, 32, FAKE, None) == _lib.KR_ERR_ALIGNMENT
+        assert f(None, 0, None, None) == 0
+
+
 def test_probe_argument_errors(lib):
     assert lib.kr_probe_read(FAKE, 24, None, None) == _lib.KR_ERR_NUMEL_MOD8
     assert lib.kr_probe_read(None, 32, None, None) == _lib.KR_ERR_NULL_POINTER

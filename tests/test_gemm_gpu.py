@@ -65,6 +65,65 @@ def test_gemm_all_reduce_shapes(dev, tile, shape, b_t):
     torch.testing.assert_close(plain.cpu(), orc.gemm_all_reduce(a, b), rtol=1e-3, atol=1e-3)
 
 
+def test_fp8_conversions(dev):
+    """kr_cast_fp8_to_bf16 on all 256 codes and kr_cast_f32_to_fp8 on random and boundary values,
+    against torch's CPU conversions (nearest even); from magnitude 448 on the result saturates to
+    448 where torch gives NaN (from 464 on)."""
+    lib = _lib.load()
+    stream = torch.cuda.current_stream(dev).cuda_stream
+    fp8 = torch.float8_e4m3fn
+    codes = torch.arange(256, dtype=torch.uint8).repeat(4)
+    out = torch.empty(codes.numel(), dtype=BF16, device=dev)
+    assert lib.kr_cast_fp8_to_bf16(codes.to(dev).data_ptr(), codes.numel(), out.data_ptr(), stream) == 0
+    want = codes.view(fp8).to(BF16)
+    nan = torch.isnan(want)
+    assert torch.equal(torch.isnan(out.cpu()), nan) and torch.equal(out.cpu()[~nan].view(torch.int16), want[~nan].view(torch.int16))
+    g = torch.Generator().manual_seed(3)
+    x = torch.cat([torch.randn(1 << 16, generator=g) * s_ for s_ in (1e-3, 0.02, 1.0, 30.0, 300.0)])
+    edge = torch.tensor([0.0, -0.0, 2.0 ** -9, 2.0 ** -10, 1.5 * 2.0 ** -9, 2.5 * 2.0 ** -9, 2.0 ** -6, 0.9375 * 2.0 ** -6,
+                         447.9, 448.0, 463.9, 464.0, 1e9, -1e9, float("inf"), -float("inf")])
+    x = torch.cat([x, edge, torch.zeros(-(x.numel() + edge.numel()) % 16)])
+    y = torch.empty(x.numel(), dtype=torch.uint8, device=dev)
+    assert lib.kr_cast_f32_to_fp8(x.to(dev).data_ptr(), x.numel(), y.data_ptr(), stream) == 0
+    got = y.cpu()
+    small = x.abs() < 448
+    assert torch.equal(got[small], x[small].to(fp8).view(torch.uint8))
+    assert torch.equal(got[~small] & 0x7f, torch.full_like(got[~small], 0x7e))           # saturated, sign kept
+    assert torch.equal(got[~small] >> 7, (x[~small] < 0).to(torch.uint8))
+    z = torch.full((16,), float("nan"))
+    assert lib.kr_cast_f32_to_fp8(z.to(dev).data_ptr(), 16, y.data_ptr(), stream) == 0
+    assert torch.isnan(y.cpu()[:16].view(fp8).float()).all()
+
+
+def test_all_gather_matmul_fp8(dev):
+    """The fp8 branch (kraken/fused/all_gather_matmul.py:53,121,213): fp8 shards and b, fp8 result.
+    With small integers and halves every fp32 sum is exact whatever its order, so the result equals
+    the oracle bit for bit, saturated elements included; with random operands it is within one fp8
+    step of the oracle (the orders of the fp32 sums differ) and mostly equal."""
+    fp8 = torch.float8_e4m3fn
+    W, m, K, N = 8, 64, 512, 384
+    g = torch.Generator().manual_seed(11)
+    a = torch.randint(-2, 3, (W, m, K), generator=g).float().to(fp8)
+    bT = (torch.randint(-3, 4, (N, K), generator=g).float() * 0.5).to(fp8)
+    a_out, c = fused.all_gather_matmul(a.to(dev), bT.to(dev).T, rank=3)
+    a_full, want = orc.all_gather_matmul_fp8(a, bT.T)
+    assert c.dtype == fp8 and a_out.dtype == fp8
+    assert torch.equal(a_out.cpu().view(torch.uint8), a_full.view(torch.uint8))
+    assert torch.equal(c.cpu().view(torch.uint8), want.view(torch.uint8))
+    # a shape the 256x256 kernel takes, random operands, one fp8 step of slack
+    W, m, K, N = 8, 512, 1024, 4096
+    a = (torch.randn(W, m, K, generator=g)).to(fp8)
+    bT = (torch.randn(N, K, generator=g) * 0.05).to(fp8)
+    _, c = fused.all_gather_matmul(a.to(dev), bT.to(dev).T)
+    _, want = orc.all_gather_matmul_fp8(a, bT.T)
+    got, ref = c.cpu().float(), want.float()
+    assert (got == ref).float().mean() > 0.99
+    step = torch.maximum(ref.abs(), torch.tensor(2.0 ** -6)) * 2.0 ** -3          # spacing of e4m3 at that magnitude
+    assert ((got - ref).abs() <= step).all()
+    with pytest.raises(NotImplementedError):
+        fused.all_gather_matmul(a.to(dev), bT.to(dev).T, gather=True)
+
+
 def test_split_fp32_is_one_pass_and_bit_exact(dev):
     """kr_split_fp32 writes the hi / lo blocks of an fp32 operand in the three layouts the GEMM
     wrappers use, bit for bit what elementwise torch ops give (hi = bf16(x), lo = bf16(x - hi)),

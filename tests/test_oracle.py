@@ -247,6 +247,51 @@ def test_all_gather_matmul_exact_gather():
     torch.testing.assert_close(c.float(), torch.cat([s.float() @ b.float() for s in stack], 0), rtol=2 ** -7, atol=1e-5)
 
 
+def test_all_gather_matmul_fp8_pins():
+    """fp8 operands, fp32 accumulate, one rounding to fp8: closed forms, saturation at 448, and for
+    random operands the nearest representable value found by searching the table of all finite
+    e4m3 codes (ties to the even code) around the product computed exactly in float64."""
+    fp8 = torch.float8_e4m3fn
+    W, m, K, N = 4, 8, 32, 16
+    # closed forms on exactly representable values: every element K * s * t
+    for s_, t_, want in ((0.5, 0.25, 4.0), (1.5, 2.0, 96.0), (2.0, 8.0, 448.0), (16.0, 16.0, 448.0), (-16.0, 16.0, -448.0)):
+        a = torch.full((W, m, K), s_).to(fp8)
+        b = torch.full((K, N), t_).to(fp8)
+        a_full, c = orc.all_gather_matmul_fp8(a, b)
+        assert c.dtype == fp8 and torch.equal(a_full.view(torch.uint8), a.reshape(W * m, K).view(torch.uint8))
+        assert torch.equal(c.float(), torch.full((W * m, N), want)), (s_, t_)
+    # the table of finite codes, by its definition: (-1)^s 2^(e-7) (1 + f/8), subnormals f/8 * 2^-6
+    vals = []
+    for code in range(256):
+        e, f = (code >> 3) & 15, code & 7
+        if e == 15 and f == 7:
+            continue
+        v = (f / 8.0) * 2.0 ** -6 if e == 0 else (1 + f / 8.0) * 2.0 ** (e - 7)
+        vals.append((-v if code & 0x80 else v, code))
+    table = torch.tensor([v for v, _ in vals], dtype=torch.float64)
+    codes = torch.tensor([c for _, c in vals])
+    assert torch.equal(codes.to(torch.uint8).view(fp8).double(), table)          # torch's decoding agrees with the definition
+    g = torch.Generator().manual_seed(5)
+    scale = torch.tensor([32.0, 2.0, 0.25, 1.0 / 64]).reshape(W, 1, 1)            # saturating, ordinary and tiny rows
+    a = (torch.randn(W, m, K, generator=g) * scale).to(fp8)
+    b = (torch.randn(K, N, generator=g) * 3).to(fp8)
+    _, c = orc.all_gather_matmul_fp8(a, b)
+    exact = a.reshape(W * m, K).double() @ b.double()                             # exact: 8-bit significands, 32 terms
+    dist = (exact.reshape(-1, 1) - table.reshape(1, -1)).abs()
+    best = dist.min(dim=1).values
+    near = dist <= best.reshape(-1, 1)                                            # one candidate, or two at a tie
+    got = c.reshape(-1).view(torch.uint8).to(torch.int64)
+    for i in range(got.numel()):
+        cand = codes[near[i]]
+        if exact.reshape(-1)[i].abs() >= 448:
+            assert (int(got[i]) & 0x7f) == 0x7e
+        elif cand.numel() == 1:
+            assert int(got[i]) == int(cand[0]) or (float(exact.reshape(-1)[i]) == 0.0 and (int(got[i]) & 0x7f) == 0)
+        else:
+            assert int(got[i]) in [int(x) for x in cand if int(x) % 2 == 0]
+    assert (exact.abs() >= 448).any() and (exact.abs() < 1).any()                # both ends of the range are exercised
+
+
 def test_known_answers_of_the_reference_tests():
     """tests/golden/known_answers.json: the closed-form cases of the reference's tests, against the oracle."""
     import json
