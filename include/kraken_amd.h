@@ -490,7 +490,9 @@ int kr_cast_f32_to_fp8(const void* src, int64_t n, void* dst, void* stream);
  *   plan[3] 256 tile: tiles of the last partial round that are split, plan[4] parts of each
  *   plan[5] column panels per scheduling group
  *   plan[6] 1: tiles that lie wholly in the reduce band add the peers on the matrix cores
- *   plan[7] 1: M or N is not a multiple of the tile (bounds-checked edge tiles)
+ *   plan[7] bit 0: M or N is not a multiple of the tile (bounds-checked edge tiles); bit 1: the
+ *           tile is 256 x 224 (a plain product with transposed-contiguous B that fills whole rounds
+ *           of the compute units with 224-column tiles and not with 256-column ones)
  */
 int kr_gemm_plan(int64_t M, int64_t N, int64_t K, int b_transposed, int n_peers, int64_t band_rows,
                  int has_bias, int has_c_full, int64_t workspace_bytes, int32_t plan[8]);

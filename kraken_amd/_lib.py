@@ -152,13 +152,15 @@ def gemm_plan(M: int, N: int, K: int, b_transposed: bool, n_peers: int = 0, band
                              int(has_bias), int(has_c_full), workspace_bytes, plan)
     check(rc, "gemm_plan")
     tile, block, splits, tail, tail_splits, group_n, mfma_peers, ragged = list(plan)
+    n224 = bool(ragged & 2)
+    ragged &= 1
     if tile == 256:
-        kernel = "gemm_dtl16_kernel" if block == 16 else "gemm_dtl_kernel"
+        kernel = "gemm_dtl16n7_kernel" if n224 else "gemm_dtl16_kernel" if block == 16 else "gemm_dtl_kernel"
     else:
         kernel = "gemm_reduce_kernel"
     return {"kernel": kernel, "tile": tile, "mfma": "16x16x32" if block == 16 else "32x32x16", "k_splits": splits,
             "tail_tiles": tail, "tail_splits": tail_splits, "group_n": group_n, "peers_on_mfma": bool(mfma_peers),
-            "ragged": bool(ragged)}
+            "ragged": bool(ragged), "tile_n": 224 if n224 else tile}
 
 
 def reload_env() -> None:

@@ -131,6 +131,7 @@ struct EnvSwitches {
     int gemm_group;      // KRAKEN_AMD_GEMM_GROUP=<n>
     int gemm_splitk;     // KRAKEN_AMD_GEMM_SPLITK=<n>
     int gemm_tailsplit;  // KRAKEN_AMD_GEMM_TAILSPLIT=<n>
+    int gemm_n224;       // KRAKEN_AMD_GEMM_N224=0|1
 };
 const EnvSwitches& env_switches();   // status.hip
 

@@ -510,9 +510,10 @@ struct GemmPlan {
     int tail_tiles;      // 256x256 kernel: tiles of the last partial round that are split ...
     int tail_splits;     // ... into this many parts each
     int splits;          // 128x128 kernel: workgroups per tile (split K loop), 1 = one pass
+    int n224;            // 256x224 tiles instead of 256x256 (whole rounds of compute units where those leave a partial one)
 };
 static GemmPlan plan_gemm(int64_t M, int64_t N, int64_t K, bool b_nt, int n_peers, int64_t band_rows, bool plain,
-                          bool has_workspace, int64_t workspace_bytes, bool has_gather, bool has_progress, bool flagged,
+                          bool plain_bf16_all_rows, bool has_workspace, int64_t workspace_bytes, bool has_gather, bool has_progress, bool flagged,
                           bool dtl_ok) {
     GemmPlan p{};
     // Tile choice: the 256x256 tile of the LDS-DMA kernel (4 waves x 128x128) has the highest
@@ -569,6 +570,24 @@ static GemmPlan plan_gemm(int64_t M, int64_t N, int64_t K, bool b_nt, int n_peer
         if (tail > 0 && gemm_dtl_tail_workspace_bytes(tail, ts) <= workspace_bytes) {
             p.tail_tiles = tail;
             p.tail_splits = ts;
+        }
+    }
+    // 256x224 tiles: a plain product (no peers, bias, band or second output; bf16 result, which the
+    // caller vouches for) with transposed-contiguous B whose columns 224 divides, when that tiling
+    // needs fewer column-units of work than 256-column tiles rounded up to whole rounds of the
+    // 256 compute units (8192 x 3584: 448 tiles = 2 rounds of 256 columns against 512 tiles = 2
+    // rounds of 224: measured 340 -> 320 us at K = 8192); a 224-column tile costs about 3 % more
+    // per flop (A is read from LDS and L2 for fewer columns).  KRAKEN_AMD_GEMM_N224=0|1 overrides.
+    p.n224 = 0;
+    if (dtl && p.mi16 && b_nt && plain && plain_bf16_all_rows && !has_gather && M % 256 == 0 && N % 224 == 0) {
+        const int64_t t8 = tiles_m * tiles_n, t7 = (M / 256) * (N / 224);
+        const double cost8 = (double)((t8 + 255) / 256) * 256.0, cost7 = (double)((t7 + 255) / 256) * 224.0 * 1.03;
+        bool use = cost7 < cost8;
+        if (env_switches().gemm_n224 >= 0) use = env_switches().gemm_n224 != 0;
+        if (use) {
+            p.n224 = 1;
+            p.tail_tiles = 0;
+            p.tail_splits = 1;
         }
     }
     // Split K loop (128x128 kernel, workspace given): with few tiles most CUs would idle, so S
@@ -689,7 +708,7 @@ static int gemm_reduce(const void* A, int64_t lda_m, int64_t lda_k, const void* 
     g.out_is_fp32 = out_is_fp32;
 
     const GemmPlan plan = plan_gemm(M, N, K, b_nt, n_peers, band_rows, n_peers == 0 && c_full == nullptr && bias == nullptr,
-                                    workspace != nullptr, workspace_bytes, gather != nullptr, g.progress != nullptr,
+                                    !out_is_fp32 && band_row0 == 0 && band_rows == M, workspace != nullptr, workspace_bytes, gather != nullptr, g.progress != nullptr,
                                     g.progress != nullptr || g.band_counter != nullptr,
                                     gemm_dtl_supported(g) && (g.a_local == nullptr || (int64_t)256 * g.lda_local * 2 < 0x7fffffffLL));
     const bool dtl = plan.tile == 256;
@@ -702,7 +721,8 @@ static int gemm_reduce(const void* A, int64_t lda_m, int64_t lda_k, const void* 
     }
     g.peers_on_mfma = plan.peers_on_mfma;
     g.mi16 = plan.mi16;
-    const int bm = plan.tile, bn = bm;
+    g.n224 = plan.n224;
+    const int bm = plan.tile, bn = plan.n224 ? 224 : bm;
     g.tiles_m = (int)((M + bm - 1) / bm);
     g.tiles_n = (int)((N + bn - 1) / bn);
     if ((int64_t)g.tiles_m * g.tiles_n > 0x7fffffffLL) return KR_ERR_BAD_DIM;
@@ -822,7 +842,7 @@ extern "C" int kr_gemm_plan(int64_t M, int64_t N, int64_t K, int b_transposed, i
     g.lda = K;
     g.ldb = b_transposed ? K : N;
     const GemmPlan p = plan_gemm(M, N, K, b_transposed != 0, n_peers, band_rows, n_peers == 0 && !has_c_full && !has_bias,
-                                 workspace_bytes > 0, workspace_bytes, false, false, false, gemm_dtl_supported(g));
+                                 band_rows == M, workspace_bytes > 0, workspace_bytes, false, false, false, gemm_dtl_supported(g));
     const bool whole_band_peers = p.tile == 256 && n_peers > 0 && p.peers_on_mfma != 0;
     plan[0] = p.tile;
     plan[1] = p.tile == 256 ? (p.mi16 ? 16 : 32) : 32;   // MFMA block rows: 16x16x32 or 32x32x16
@@ -832,6 +852,7 @@ extern "C" int kr_gemm_plan(int64_t M, int64_t N, int64_t K, int b_transposed, i
     plan[5] = p.group_n;
     plan[6] = whole_band_peers ? 1 : 0;
     plan[7] = (M % p.tile != 0 || N % p.tile != 0) ? 1 : 0;
+    if (p.n224) plan[7] |= 2;   // bit 1: 256 x 224 tiles
     return KR_OK;
 }
 

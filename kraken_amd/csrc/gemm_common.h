@@ -40,7 +40,8 @@ struct GemmArgs {
     int tail_tiles;
     int group_n;         // column panels per scheduling group (tile_schedule)
     int peers_on_mfma;   // 256x256 kernel: add whole-band tiles' peers through the matrix cores
-    int mi16;            // 256x256 kernel: k loop on 16x16x32 MFMA blocks (peers in the epilogue)
+    int mi16;            // 256x256 kernel: k loop and peer phase on 16x16x32 MFMA blocks
+    int n224;            // 256x224 tiles (tiles_n counts them): plain product, transposed-contiguous B, whole rounds
     // producer of the copy-engine reduce-scatter (band_counter == nullptr: off): finished tiles are
     // counted per destination rank, whose band is count_rows rows of C
     uint32_t* band_counter;   // [M / count_rows] tiles finished that touch the band

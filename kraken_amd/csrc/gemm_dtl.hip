@@ -57,6 +57,43 @@ typedef __attribute__((address_space(3))) s16x4* lds_tr;
 constexpr int vmcnt_imm(int n) { return (n & 15) | (7 << 4) | (15 << 8) | ((n >> 4) << 14); }
 constexpr int kLgkm0 = 0xc07f;   // s_waitcnt lgkmcnt(0) only
 
+// bf16 store of a wave's 128 x (NB*16) part of a tile held as 8 x NB accumulator blocks of 16 x 16
+// (lane l: row l%16, columns 4(l/16) .. +3 of a block): per 16-row slab the blocks are rounded to
+// bf16 into a per-wave LDS patch [16][NB*16 + 8] and leave as 16-byte chunks of whole rows.
+// `smem`: the workgroup's LDS, free for reuse; `dst`: the wave's first row and column; ld in elements.
+template <int NB>
+__device__ __forceinline__ void store_tile_bf16_blocks(const f32x4 (&acc16)[2 * TM][NB], unsigned char* smem, uint16_t* dst, int64_t ld,
+                                                       int lane, int wave) {
+    constexpr int COLS = NB * 16, LD = COLS + 8, CPR = COLS / 8, CHUNKS = 16 * CPR;
+    static_assert(16 * LD * 2 <= 4096, "patch of a wave");
+    uint16_t* patch = (uint16_t*)(smem + wave * 4096);
+    typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+#pragma unroll
+    for (int i = 0; i < 2 * TM; ++i) {
+#pragma unroll
+        for (int j = 0; j < NB; ++j) {
+            // (pinned here: a conversion the compiler may hoist would keep all blocks' halves alive at once)
+            uint32_t lo, hi, t;
+            asm volatile("v_accvgpr_read_b32 %0, %2\n\tv_accvgpr_read_b32 %1, %3\n\tv_cvt_pk_bf16_f32 %0, %0, %1"
+                         : "=&v"(lo), "=&v"(t) : "a"(acc16[i][j][0]), "a"(acc16[i][j][1]));
+            asm volatile("v_accvgpr_read_b32 %0, %2\n\tv_accvgpr_read_b32 %1, %3\n\tv_cvt_pk_bf16_f32 %0, %0, %1"
+                         : "=&v"(hi), "=&v"(t) : "a"(acc16[i][j][2]), "a"(acc16[i][j][3]));
+            *(u32x2*)(patch + (lane & 15) * LD + 16 * j + 4 * (lane >> 4)) = u32x2{lo, hi};
+        }
+        asm volatile("" ::: "memory");   // the reads below see the stores above (different vector types, same bytes)
+#pragma unroll
+        for (int it = 0; it < (CHUNKS + 63) / 64; ++it) {
+            const int idx = it * 64 + lane;
+            if (idx < CHUNKS) {
+                const int r = idx / CPR, c = idx - r * CPR;
+                const u32x4 v = *(const u32x4*)(patch + r * LD + c * 8);
+                st_stream((u32x4*)(dst + (int64_t)(16 * i + r) * ld + c * 8), v);
+            }
+        }
+        asm volatile("" ::: "memory");   // the next slab's stores stay behind these reads
+    }
+}
+
 // One workgroup tile.  PEERS_FIRST picks the order of the two accumulation phases (peers'
 // partial sums, k loop) for tiles whose peers are added on the matrix cores.
 // SPLIT: the workgroup is one of g.k_splits that share a tile of the last partial round: it
@@ -66,8 +103,18 @@ constexpr int kLgkm0 = 0xc07f;   // s_waitcnt lgkmcnt(0) only
 // 32x32x16 (4 x 4 blocks of 32 x 32): same operand traffic, but the matrix cores draw less power
 // per flop with it (under the power limit, matrix-core-only loops on random operands sustain
 // 2.04 PFLOP/s with 16x16x32 against 1.62 with 32x32x16).
-template <bool B_NT, bool PEERS_FIRST, bool SPLIT = false, bool RAGGED = false, bool MI16 = false>
+// NB: 16-column blocks per wave (16x16 form).  8 = the 256 x 256 tile; 7 = a 256 x 224 tile (waves of
+// 128 x 112) for plain products with transposed-contiguous B whose 256-column tiles would leave a
+// partial last round of compute units while 224-column tiles fill whole rounds (8192 x 3584: 448
+// tiles = 1.75 rounds against 512 = 2).  Per flop the narrower tile reads 7 % more of A from LDS
+// and L2, which two full rounds more than pay for.
+template <bool B_NT, bool PEERS_FIRST, bool SPLIT = false, bool RAGGED = false, bool MI16 = false, int NB = 2 * TN>
 __device__ __forceinline__ void gemm_dtl_tile(const GemmArgs& g, unsigned char* smem) {
+    static_assert(NB == 2 * TN || (NB == 7 && MI16 && B_NT && !SPLIT && !RAGGED && !PEERS_FIRST), "224-column tile: plain NT products only");
+    constexpr int BNX = WN * NB * 16;                            // columns of the workgroup tile
+    constexpr int WTNX = NB * 16;                                // columns of a wave
+    constexpr int LOADS_B = BNX * BKD * 2 / 1024 / (WM * WN);    // LDS-DMA loads of B per wave per k-step: 8 or 7
+    constexpr int LOADS_TILE = LOADS_A + LOADS_B;
     // Nothing is outstanding at kernel entry; saying so keeps the compiler's own wait-count
     // bookkeeping from carrying the pending loads and stores of the other copy of this code
     // (which never runs in the same workgroup) into this one, where it cannot see the LDS-DMA
@@ -84,7 +131,7 @@ __device__ __forceinline__ void gemm_dtl_tile(const GemmArgs& g, unsigned char* 
     const int tail_index = SPLIT ? (int)(blockIdx.x / (unsigned)g.k_splits) : 0;
     tile_schedule(g, SPLIT ? schedule_position(g, tail_index, first_tile) : schedule_position(g, blockIdx.x), tile_m,
                   tile_n);
-    const int m0 = tile_m * BM, n0 = tile_n * BN;
+    const int m0 = tile_m * BM, n0 = tile_n * BNX;
     // k-steps of this workgroup: all of them, or the split's share
     const int kt_all = g.K / BKD;
     const int kt_begin = SPLIT ? (int)((int64_t)kt_all * split / g.k_splits) : 0;
@@ -236,7 +283,7 @@ __device__ __forceinline__ void gemm_dtl_tile(const GemmArgs& g, unsigned char* 
 #pragma unroll
         for (int ks2 = 0; ks2 < 2; ++ks2) {
             fa16[ks2] = (uint32_t)((wm * WTM + p) * 128 + (((4 * ks2 + gq) ^ sw16) << 4));
-            if (B_NT) fb16[ks2] = B_BASE + (uint32_t)((wn * WTN + p) * 128 + (((4 * ks2 + gq) ^ sw16) << 4));
+            if (B_NT) fb16[ks2] = B_BASE + (uint32_t)((wn * WTNX + p) * 128 + (((4 * ks2 + gq) ^ sw16) << 4));
         }
         if (!B_NT) {
 #pragma unroll
@@ -273,7 +320,7 @@ __device__ __forceinline__ void gemm_dtl_tile(const GemmArgs& g, unsigned char* 
     const int band_lo = g.band_row0;
     const bool full_tile = !RAGGED || (m0 + BM <= g.M && n0 + BN <= g.N);
     const bool tile_in_band = full_tile && m0 >= band_lo && m0 + BM <= band_lo + g.band_rows;
-    const bool mfma_peers = !SPLIT && g.peers_on_mfma && g.n_peers > 0 && tile_in_band;
+    const bool mfma_peers = !SPLIT && NB == 2 * TN && g.peers_on_mfma && g.n_peers > 0 && tile_in_band;
     const bool bias_in_acc = !SPLIT && g.bias != nullptr && tile_in_band && (g.n_peers == 0 || mfma_peers);
     f32x16 acc[TM][TN];
     {
@@ -303,16 +350,16 @@ __device__ __forceinline__ void gemm_dtl_tile(const GemmArgs& g, unsigned char* 
     }
 
     // the same for the 16x16 blocks: a lane holds row lane%16 and the columns 16j + 4(lane/16) .. +3
-    f32x4 acc16[2 * TM][2 * TN];
+    f32x4 acc16[2 * TM][NB];
     if constexpr (MI16) {
-        f32x4 init16[2 * TN];
+        f32x4 init16[NB];
 #pragma unroll
-        for (int j = 0; j < 2 * TN; ++j) init16[j] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+        for (int j = 0; j < NB; ++j) init16[j] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
         if (bias_in_acc) {
             typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
-            const uint16_t* bp = g.bias + n0 + wn * WTN + 4 * (lane >> 4);
+            const uint16_t* bp = g.bias + n0 + wn * WTNX + 4 * (lane >> 4);
 #pragma unroll
-            for (int j = 0; j < 2 * TN; ++j) {
+            for (int j = 0; j < NB; ++j) {
                 const u32x2 b4 = *(const u32x2*)(bp + j * 16);
                 init16[j] = f32x4{bf16_lo(b4.x), bf16_hi(b4.x), bf16_lo(b4.y), bf16_hi(b4.y)};
             }
@@ -320,7 +367,7 @@ __device__ __forceinline__ void gemm_dtl_tile(const GemmArgs& g, unsigned char* 
 #pragma unroll
         for (int i = 0; i < 2 * TM; ++i)
 #pragma unroll
-            for (int j = 0; j < 2 * TN; ++j) acc16[i][j] = init16[j];
+            for (int j = 0; j < NB; ++j) acc16[i][j] = init16[j];
     }
 
 #define KR_SCHED_FENCE() __builtin_amdgcn_sched_barrier(0)
@@ -416,6 +463,7 @@ __device__ __forceinline__ void gemm_dtl_tile(const GemmArgs& g, unsigned char* 
     // 32x32x16 form.  An odd peer count repeats the last peer as b and masks it in X (a product
     // 0 * finite adds nothing).
     auto peer_phase16 = [&]() __attribute__((always_inline)) {
+        if constexpr (NB == 2 * TN) {
         constexpr int kItemLoads = 8;
         constexpr int kItemBytes = kItemLoads * 1024;
         constexpr int kAhead = 4;
@@ -492,6 +540,7 @@ __device__ __forceinline__ void gemm_dtl_tile(const GemmArgs& g, unsigned char* 
         }
         __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));
         __syncthreads();   // the ring is handed on (k loop or epilogue patches of other waves)
+        }
     };
     // An empty statement that names every accumulator as an AGPR operand, placed between the
     // phases: with the live ranges cut here the register allocator keeps the accumulators
@@ -501,7 +550,7 @@ __device__ __forceinline__ void gemm_dtl_tile(const GemmArgs& g, unsigned char* 
 #pragma unroll
             for (int i = 0; i < 2 * TM; ++i)
 #pragma unroll
-                for (int j = 0; j < 2 * TN; ++j) asm volatile("" : "+a"(acc16[i][j]));
+                for (int j = 0; j < NB; ++j) asm volatile("" : "+a"(acc16[i][j]));
         } else {
 #pragma unroll
             for (int i = 0; i < TM; ++i)
@@ -510,8 +559,8 @@ __device__ __forceinline__ void gemm_dtl_tile(const GemmArgs& g, unsigned char* 
         }
     };
     if (PEERS_FIRST && mfma_peers) {
-        if constexpr (MI16) peer_phase16();
-        else peer_phase();
+        if constexpr (MI16 && NB == 2 * TN) peer_phase16();
+        else if constexpr (!MI16) peer_phase();
     }
     pin_accumulators();
 
@@ -525,10 +574,11 @@ __device__ __forceinline__ void gemm_dtl_tile(const GemmArgs& g, unsigned char* 
     // has half as many MFMAs to hide behind; there 14 loads of step t+2 go out behind the barrier
     // of step t, one per four MFMAs -- 64 cycles apart, as above -- and the last two at the start
     // of step t+1)
-    constexpr int kEarly = MI16 ? 14 : 6;
-    static_assert(NSTAGE == 2 && LOADS_PER_TILE == 16, "load schedule below: 6 + 8 + 2 loads");
+    // (224-column tile: 15 loads per k-step and 56 MFMAs per sub-step: 12 behind the barrier, 3 at the start)
+    constexpr int kEarly = MI16 ? (NB == 7 ? 12 : 14) : 6;
+    static_assert(NSTAGE == 2 && LOADS_PER_TILE == 16 && (LOADS_TILE == 16 || (NB == 7 && LOADS_TILE == 15)), "load schedule below: 6 + 8 + 2 loads");
 #pragma unroll
-    for (int q = 0; q < LOADS_PER_TILE; ++q) issue_load(0, 0, q);
+    for (int q = 0; q < LOADS_TILE; ++q) issue_load(0, 0, q);
 #pragma unroll
     for (int q = 0; q < kEarly; ++q) issue_load(1, 1, q);
     __builtin_amdgcn_s_waitcnt(vmcnt_imm(kEarly));
@@ -536,7 +586,7 @@ __device__ __forceinline__ void gemm_dtl_tile(const GemmArgs& g, unsigned char* 
     KR_SCHED_FENCE();
     if constexpr (MI16) {   // (A blocks 4..7 are read inside the first sub-step)
 #pragma unroll
-        for (int j = 0; j < 2 * TN; ++j) read_b16(0, j, 0, 0);
+        for (int j = 0; j < NB; ++j) read_b16(0, j, 0, 0);
 #pragma unroll
         for (int i = 0; i < TM; ++i) read_a16(0, i, 0, 0);
     } else {
@@ -602,15 +652,18 @@ __device__ __forceinline__ void gemm_dtl_tile(const GemmArgs& g, unsigned char* 
     // Two barriers instead of one buy the loads a third more time to arrive (from slot 9 of one
     // step to slot 47 of the next): the wait sits right in front of the first read that needs
     // the data, not in front of the first load that needs the room.
-    constexpr int NM16 = 4 * TM * TN;
+    // (224-column tile, NB = 7: 56 MFMAs per sub-step; everything keeps its distance from the end of
+    // the sub-step: barrier (a) behind MFMA 6, barrier (b) behind MFMA 39, the same 16 slots behind it
+    // for the 7 + 4 fragments of the next step; 15 fragments of sub-step 1 to read in sub-step 0)
+    constexpr int NM16 = 2 * TM * NB;
     auto read_frag16 = [&](int buf, int r, int ks2, uint32_t stage_off) __attribute__((always_inline)) {
-        if (r < 2 * TN) read_b16(buf, r, ks2, stage_off);
-        else read_a16(buf, r - 2 * TN, ks2, stage_off);
+        if (r < NB) read_b16(buf, r, ks2, stage_off);
+        else read_a16(buf, r - NB, ks2, stage_off);
     };
-    constexpr int kBarA = 2 * TN - 1;      // last MFMA of the first row
-    constexpr int kBarB = 47;
+    constexpr int kBarA = NB - 1;          // last MFMA of the first row
+    constexpr int kBarB = NM16 - 17;
     constexpr int kLoadsBeforeB = (kBarB - kBarA - 2) / 4 + 1;   // loads of step t+2 in slots 9, 13, ... < kBarB
-    static_assert(!MI16 || (kLoadsBeforeB == 10 && kLoadsBeforeB <= kEarly), "wait count of barrier (b)");
+    static_assert(!MI16 || ((kLoadsBeforeB == 10 || (NB == 7 && kLoadsBeforeB == 8)) && kLoadsBeforeB <= kEarly), "wait count of barrier (b)");
     auto k_step16 = [&](int t, auto stage_c) __attribute__((always_inline)) {
         const uint32_t stage_cur = stage_c;
         const uint32_t stage_nxt = stage_cur ^ 1u;
@@ -620,7 +673,7 @@ __device__ __forceinline__ void gemm_dtl_tile(const GemmArgs& g, unsigned char* 
             const int cur = ks2, nxt = cur ^ 1;
 #pragma unroll
             for (int s = 0; s < NM16; ++s) {
-                const int i = s / (2 * TN), j = s % (2 * TN);
+                const int i = s / NB, j = s % NB;
                 // (written out with the accumulator tied to the AGPRs it lives in: given the
                 // builtin, the register allocator moves accumulators through VGPRs and other
                 // AGPRs around the MFMAs, a copy or two per MFMA)
@@ -629,9 +682,10 @@ __device__ __forceinline__ void gemm_dtl_tile(const GemmArgs& g, unsigned char* 
                              : "v"(bfr16[cur][j]), "v"(af16[cur][i]));
                 if (ks2 == 0) {
                     if (s % 4 == 0) read_frag16(nxt, s / 4, 1, st_cur);
+                    if (NB == 7 && s == NM16 - 3) read_frag16(nxt, NB + 2 * TM - 1, 1, st_cur);   // the fifteenth
                     if (s % 8 == 1 && s / 8 + 4 < 2 * TM) read_a16(cur, s / 8 + 4, 0, st_cur);
                     // the last loads of step t+1
-                    if ((s == 2 || s == 6) && kEarly + s / 4 < LOADS_PER_TILE) issue_load(t + 1, stage_nxt, kEarly + s / 4);
+                    if (s % 4 == 2 && s < 16 && kEarly + s / 4 < LOADS_TILE) issue_load(t + 1, stage_nxt, kEarly + s / 4);
                 } else {
                     if (s == kBarA) {
                         KR_SCHED_FENCE();
@@ -647,8 +701,8 @@ __device__ __forceinline__ void gemm_dtl_tile(const GemmArgs& g, unsigned char* 
                     }
                     // B blocks and A blocks 0..3 of k-step t+1: slots 48, 50, ..., 62; 63; 51, 55, 59
                     if (s > kBarB && s % 2 == 0) read_frag16(nxt, (s - kBarB - 1) / 2, 0, st_nxt);
-                    if (s == NM16 - 1) read_frag16(nxt, 2 * TN, 0, st_nxt);
-                    if (s > kBarB && s % 4 == 3 && s < NM16 - 1) read_frag16(nxt, 2 * TN + 1 + (s - kBarB - 4) / 4, 0, st_nxt);
+                    if (NB == 2 * TN && s == NM16 - 1) read_frag16(nxt, NB, 0, st_nxt);   // (NB = 7: A block 0 came with slot 54)
+                    if (s > kBarB && s % 4 == 3 && s < NM16 - 1) read_frag16(nxt, NB + 1 + (s - kBarB - 4) / 4, 0, st_nxt);
                 }
                 KR_SCHED_FENCE();
             }
@@ -704,12 +758,15 @@ __device__ __forceinline__ void gemm_dtl_tile(const GemmArgs& g, unsigned char* 
         return;
     }
     if (!PEERS_FIRST && mfma_peers) {
-        if constexpr (MI16) peer_phase16();
-        else peer_phase();
+        if constexpr (MI16 && NB == 2 * TN) peer_phase16();
+        else if constexpr (!MI16) peer_phase();
     }
     pin_accumulators();
     // peers and bias that are already in the accumulators are not added again
-    if constexpr (MI16) {
+    if constexpr (NB != 2 * TN) {
+        // 224-column tile of a plain product: every row goes to `out`
+        store_tile_bf16_blocks<NB>(acc16, smem, (uint16_t*)g.out + (int64_t)(m0 + wm * WTM) * g.N + n0 + wn * WTNX, g.N, lane, wave);
+    } else if constexpr (MI16) {
         if (full_tile) {
             gemm_epilogue<BM, WTM, WTN, TM, TN, true, EP_WAVE>(g, mfma_peers ? 0 : g.n_peers, bias_in_acc ? nullptr : g.bias, acc16,
                                                                smem, m0, n0, wm, wn, lane, wave);
@@ -741,6 +798,12 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_dtl16_kernel(const GemmArgs 
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     if (g.peers_on_mfma && g.n_peers > 0 && (g.peers_on_mfma == 1 ? ((blockIdx.x >> 3) & 1) : g.peers_on_mfma == 2)) gemm_dtl_tile<B_NT, true, false, RAGGED, true>(g, smem);
     else gemm_dtl_tile<B_NT, false, false, RAGGED, true>(g, smem);
+}
+
+// 256 x 224 tiles (plain products, transposed-contiguous B).
+__global__ __launch_bounds__(WM* WN * 64) void gemm_dtl16n7_kernel(const GemmArgs g) {
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+    gemm_dtl_tile<true, false, false, false, true, 7>(g, smem);
 }
 
 }  // namespace
@@ -834,6 +897,12 @@ hipError_t launch_gemm_dtl(const GemmArgs& g, bool b_nt, hipStream_t st, void* w
     static std::atomic<uint64_t> opted[8];
     if (hipError_t e = lds_opt_in(kfn, LDS_BYTES, opted[(g.mi16 ? 4 : 0) + (b_nt ? 2 : 0) + (ragged ? 1 : 0)]); e != hipSuccess)
         return e;
+    if (g.n224) {
+        static std::atomic<uint64_t> nopted;
+        if (hipError_t e = lds_opt_in((const void*)gemm_dtl16n7_kernel, LDS_BYTES, nopted); e != hipSuccess) return e;
+        hipLaunchKernelGGL(gemm_dtl16n7_kernel, grid, block, LDS_BYTES, st, g);
+        return hipGetLastError();
+    }
     if (grid.x == 0) {
         // every tile belongs to the split partial round
     } else if (g.mi16) {

@@ -21,6 +21,7 @@ static EnvSwitches read_env() {
     e.gemm_group = num("KRAKEN_AMD_GEMM_GROUP");
     e.gemm_splitk = num("KRAKEN_AMD_GEMM_SPLITK");
     e.gemm_tailsplit = num("KRAKEN_AMD_GEMM_TAILSPLIT");
+    e.gemm_n224 = num("KRAKEN_AMD_GEMM_N224");
     return e;
 }
 static EnvSwitches& env_storage() {

@@ -300,8 +300,14 @@ def test_gemm_plan_reports_the_dispatch(lib, monkeypatch):
     assert p["kernel"] == "gemm_dtl16_kernel" and p["tile"] == 256 and p["mfma"] == "16x16x32" and p["peers_on_mfma"]
     p = _lib.gemm_plan(4096, 8192, 1024, False, 7, 4096, True, False)        # every tile streams peers
     assert p["kernel"] == "gemm_dtl16_kernel" and p["mfma"] == "16x16x32" and p["peers_on_mfma"] and p["group_n"] == 16
-    p = _lib.gemm_plan(8192, 3584, 8192, True)                               # all-gather matmul shape
-    assert p["kernel"] == "gemm_dtl16_kernel" and p["group_n"] == 4 and p["tail_tiles"] == 0
+    p = _lib.gemm_plan(8192, 3584, 8192, True)                               # all-gather matmul shape: 448 tiles of 256 columns
+    assert p["kernel"] == "gemm_dtl16n7_kernel" and p["tile_n"] == 224 and p["group_n"] == 4 and p["tail_tiles"] == 0   # 512 of 224
+    assert _lib.gemm_plan(8192, 3584, 8192, False)["tile_n"] == 256          # row-major B: no 224-column form
+    assert _lib.gemm_plan(8192, 3584, 8192, True, 7, 8192)["tile_n"] == 256  # peers: not a plain product
+    assert _lib.gemm_plan(8192, 3584, 8192, True, has_bias=True)["tile_n"] == 256
+    assert _lib.gemm_plan(8192, 7168, 4096, True)["tile_n"] == 224           # 896 tiles = 3.5 rounds against 1024 = 4 rounds of 224
+    assert _lib.gemm_plan(8192, 14336, 4096, True)["tile_n"] == 256          # 1792 tiles = 7 whole rounds already
+    assert _lib.gemm_plan(8192, 4096, 8192, True)["tile_n"] == 256           # 224 does not divide N
     p = _lib.gemm_plan(256, 256, 100 * 8, False)                             # K not a multiple of 64
     assert p["kernel"] == "gemm_reduce_kernel" and p["tile"] == 128 and p["k_splits"] == 1
     need = lib.kr_gemm_workspace_bytes(128, 6656, 4096)
@@ -319,7 +325,7 @@ def test_gemm_plan_reports_the_dispatch(lib, monkeypatch):
     monkeypatch.setenv("KRAKEN_AMD_GEMM_MFMA", "32")
     _lib.reload_env()
     try:
-        assert _lib.gemm_plan(8192, 3584, 8192, True)["kernel"] == "gemm_dtl_kernel"
+        assert _lib.gemm_plan(8192, 4096, 8192, True)["kernel"] == "gemm_dtl_kernel"
     finally:
         monkeypatch.delenv("KRAKEN_AMD_GEMM_MFMA")
         _lib.reload_env()

@@ -65,6 +65,35 @@ def test_gemm_all_reduce_shapes(dev, tile, shape, b_t):
     torch.testing.assert_close(plain.cpu(), orc.gemm_all_reduce(a, b), rtol=1e-3, atol=1e-3)
 
 
+def test_all_gather_matmul_224_column_tiles(dev, monkeypatch):
+    """A plain product with transposed-contiguous B whose 256-column tiles leave a partial round of
+    compute units takes 256 x 224 tiles (4096 x 3584: 224 tiles against 256): the whole matrix against
+    the oracle, and the same bits as the 256-column form (every element sums the same products in the
+    same order)."""
+    W, m, K, N = 8, 512, 320, 3584
+    assert _lib.gemm_plan(W * m, N, K, True)["kernel"] == "gemm_dtl16n7_kernel"
+    stack = orc.make_stack(W, (m, K), seed0=21)
+    bT = orc.randn_bf16((N, K), 22, 0.05)
+    a_out, c = fused.all_gather_matmul(stack.to(dev), bT.to(dev).T, rank=5)
+    _, want = orc.all_gather_matmul(stack, bT.T)
+    torch.testing.assert_close(c.cpu().float(), want.float(), **TOL)
+    assert torch.equal(a_out.cpu(), stack.reshape(W * m, K))
+    monkeypatch.setenv("KRAKEN_AMD_GEMM_N224", "0")
+    assert _lib.gemm_plan(W * m, N, K, True)["kernel"] == "gemm_dtl16_kernel"
+    _, c256 = fused.all_gather_matmul(stack.to(dev), bT.to(dev).T, rank=5)
+    assert torch.equal(c, c256)
+    # forced on where the rule would not pick it (64 tiles of 224 columns: one partial round either way), odd k-step count
+    monkeypatch.setenv("KRAKEN_AMD_GEMM_N224", "1")
+    monkeypatch.setenv("KRAKEN_AMD_GEMM_TILE", "256")
+    W, m, K, N = 4, 256, 192, 896
+    stack = orc.make_stack(W, (m, K), seed0=23)
+    bT = orc.randn_bf16((N, K), 24, 0.05)
+    assert _lib.gemm_plan(W * m, N, K, True)["kernel"] == "gemm_dtl16n7_kernel"
+    _, c = fused.all_gather_matmul(stack.to(dev), bT.to(dev).T)
+    _, want = orc.all_gather_matmul(stack, bT.T)
+    torch.testing.assert_close(c.cpu().float(), want.float(), **TOL)
+
+
 def test_fp8_conversions(dev):
     """kr_cast_fp8_to_bf16 on all 256 codes and kr_cast_f32_to_fp8 on random and boundary values,
     against torch's CPU conversions (nearest even); from magnitude 448 on the result saturates to
