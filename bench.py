@@ -75,7 +75,7 @@ MEASURED_TRAFFIC = {
     # last-level cache, not by HBM) + write-backs
     "gemm_reduce_scatter_8192x8192x3584_w8": (985098980, "8eb5098"),    # profiles/gemm_dtl16_kernel_reduce_scatter_8192x8192x3584.md
     "gemm_all_reduce_4096x8192x1024_w8": (708000078, "8eb5098"),        # profiles/gemm_dtl16_kernel_all_reduce_4096x8192x1024.md
-    "all_gather_matmul_8192x3584x8192_w8": (876206400, "8eb5098"),      # profiles/gemm_dtl16_kernel_all_gather_matmul_8192x3584x8192.md
+    "all_gather_matmul_8192x3584x8192_w8": (837225331, "7e7356c"),      # profiles/gemm_dtl16n7_kernel_all_gather_matmul_8192x3584x8192.md
     "all_gather_matmul_4096x6656x16384_w8": (1816571183, "8eb5098"),    # profiles/gemm_dtl16_kernel_all_gather_matmul_4096x6656x16384.md
 }
 
