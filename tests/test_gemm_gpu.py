@@ -70,6 +70,8 @@ def test_all_gather_matmul_224_column_tiles(dev, monkeypatch):
     compute units takes 256 x 224 tiles (4096 x 3584: 224 tiles against 256): the whole matrix against
     the oracle, and the same bits as the 256-column form (every element sums the same products in the
     same order)."""
+    for name in ("TILE", "MFMA", "N224", "PEERS"):   # the rule under test, whatever the caller's environment forces
+        monkeypatch.delenv("KRAKEN_AMD_GEMM_" + name, raising=False)
     W, m, K, N = 8, 512, 320, 3584
     assert _lib.gemm_plan(W * m, N, K, True)["kernel"] == "gemm_dtl16n7_kernel"
     stack = orc.make_stack(W, (m, K), seed0=21)
