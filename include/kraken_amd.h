@@ -478,6 +478,22 @@ int kr_cast_fp8_to_bf16(const void* src, int64_t n, void* dst, void* stream);
 int kr_cast_f32_to_fp8(const void* src, int64_t n, void* dst, void* stream);
 
 /*
+ * out[M, N] = A[M, K] @ Bt[N, K]^T on fp8 (e4m3fn) operands with fp32 accumulation, on the fp8
+ * matrix-core instruction (v_mfma_f32_16x16x128_f8f6f4): the product of the fp8 branch of
+ * kraken/fused/all_gather_matmul.py:53,121,213 (tl.dot of float8e4nv tiles, fp32 accumulator,
+ * result cast to the operands' type) at twice the bf16 rate, without widening the operands.
+ *   A: row-major, lda bytes between rows; Bt: the right operand transposed (k contiguous), ldb
+ *   bytes between its rows -- the layout the reference's benchmark passes (`b.T` of an [N, K] tensor).
+ *   out_kind: 0 = bf16, 1 = fp32, 2 = fp8 (e4m3fn; fp32 sums rounded once, nearest even, magnitudes
+ *   from 448 on give +-448, NaN stays NaN -- the conversion of kr_cast_f32_to_fp8); out is [M, N]
+ *   contiguous.
+ * M % 256 == 0, N % 256 == 0, K % 128 == 0 (other shapes: convert with kr_cast_fp8_to_bf16 and use the
+ * bf16 entry points); lda, ldb >= K and multiples of 16; pointers 16-byte aligned.
+ */
+int kr_gemm_fp8(const void* A, int64_t lda, const void* Bt, int64_t ldb, int64_t M, int64_t N, int64_t K,
+                void* out, int out_kind, void* stream);
+
+/*
  * Which kernel kr_gemm_reduce_*_bf16 would run for a shape (contiguous operands), decided by the
  * same code that launches it; for benchmarks and logs that want to name the kernel they timed.
  * No counterpart in the reference (its tile sizes are keyword arguments of the wrappers,

@@ -706,6 +706,7 @@ static int gemm_reduce(const void* A, int64_t lda_m, int64_t lda_k, const void* 
     g.c_full = (uint16_t*)c_full;
     g.out = out;
     g.out_is_fp32 = out_is_fp32;
+    g.out_fp8 = 0;
 
     const GemmPlan plan = plan_gemm(M, N, K, b_nt, n_peers, band_rows, n_peers == 0 && c_full == nullptr && bias == nullptr,
                                     !out_is_fp32 && band_row0 == 0 && band_rows == M, workspace != nullptr, workspace_bytes, gather != nullptr, g.progress != nullptr,
@@ -827,6 +828,42 @@ extern "C" int kr_gemm_producer_bf16(const void* A, int64_t lda_m, int64_t lda_k
     // no reduce band: every row of C goes to `C`; tile order rotated to the band of rank + 1
     return gemm_reduce(A, lda_m, lda_k, B, ldb_k, ldb_n, M, N, K, nullptr, 0, nullptr, 0, nullptr, 0, 0, C, nullptr,
                        0, ((int64_t)(rank + 1) % W) * (M / W), stream, &ps);
+}
+
+// Plain product of fp8 (e4m3fn) operands on the fp8 matrix-core instruction (all_gather_matmul.py:53,121,213: fp8 shards and
+// weight, fp8 result).  The kernel is the 256x256 LDS-DMA kernel with its k-step on 16x16x128 blocks; it reads the operands
+// as matrices of two-byte units, hence the halved K and row strides below.
+extern "C" int kr_gemm_fp8(const void* A, int64_t lda, const void* Bt, int64_t ldb, int64_t M, int64_t N, int64_t K,
+                           void* out, int out_kind, void* stream) {
+    if (M < 0 || N < 0 || K < 0 || M > 0x7fffffffLL || N > 0x7fffffffLL || K > 0x7fffffffLL) return KR_ERR_BAD_DIM;
+    if (out_kind < 0 || out_kind > 2) return KR_ERR_BAD_DIM;
+    if (M % 256 != 0 || N % 256 != 0 || K % 128 != 0) return KR_ERR_BAD_DIM;
+    if (M == 0 || N == 0) return KR_OK;
+    if (K == 0) return KR_ERR_BAD_DIM;
+    if (A == nullptr || Bt == nullptr || out == nullptr) return KR_ERR_NULL_POINTER;
+    if (lda < K || ldb < K) return KR_ERR_LAYOUT;
+    if (lda % 16 != 0 || ldb % 16 != 0 || !aligned16(A) || !aligned16(Bt) || !aligned16(out)) return KR_ERR_ALIGNMENT;
+    GemmArgs g{};
+    peer_tab_stacked(g.peer, A, 0, 0);
+    g.A = (const uint16_t*)A;
+    g.B = (const uint16_t*)Bt;
+    g.lda = lda / 2;
+    g.ldb = ldb / 2;
+    g.M = (int)M; g.N = (int)N; g.K = (int)(K / 2);
+    if (!gemm_dtl_supported(g)) return KR_ERR_LAYOUT;
+    g.comm_rows = 1;
+    g.count_rows = 1;
+    g.band_row0 = 0;
+    g.band_rows = (int)M;
+    g.out = out;
+    g.out_is_fp32 = out_kind == 1;
+    g.out_fp8 = out_kind == 2;
+    g.tiles_m = (int)(M / 256);
+    g.tiles_n = (int)(N / 256);
+    g.group_n = env_switches().gemm_group > 0 ? env_switches().gemm_group : 4;
+    g.k_splits = 1;
+    g.mi16 = 1;
+    return (int)launch_gemm_dtl8(g, (hipStream_t)stream);
 }
 
 extern "C" int kr_gemm_plan(int64_t M, int64_t N, int64_t K, int b_transposed, int n_peers, int64_t band_rows,

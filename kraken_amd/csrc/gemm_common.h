@@ -21,6 +21,7 @@ struct GemmArgs {
     uint16_t* c_full;
     void* out;
     int out_is_fp32;
+    int out_fp8;       // fp8 kernel only: the result is fp8 (e4m3fn), [M, N] bytes
     int pivot_tiles;   // rotation of the M-tile order
     int tiles_m, tiles_n;
     // all-gather matmul with arrival flags (progress == nullptr: A is complete, nothing waits)
@@ -66,6 +67,7 @@ inline hipError_t lds_opt_in(const void* fn, int bytes, std::atomic<uint64_t>& d
 // LDS-DMA kernel for shapes the 256x256 tile divides (gemm_dtl.hip)
 bool gemm_dtl_supported(const GemmArgs& g);
 hipError_t launch_gemm_dtl(const GemmArgs& g, bool b_nt, hipStream_t st, void* workspace);
+hipError_t launch_gemm_dtl8(const GemmArgs& g, hipStream_t st);   // fp8 operands (gemm_dtl.hip)
 
 constexpr int kXcds = 8;
 

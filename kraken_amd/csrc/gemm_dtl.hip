@@ -94,6 +94,47 @@ __device__ __forceinline__ void store_tile_bf16_blocks(const f32x4 (&acc16)[2 * 
     }
 }
 
+// fp32 -> fp8 (e4m3fn) of two values into one half of a word: nearest even; magnitudes from 448 on
+// (infinities included) give +-448, NaN stays NaN -- the conversion kr_cast_f32_to_fp8 defines.  The
+// clamp is explicit, so the instruction's own overflow handling never comes into play.
+template <bool HIGH_HALF>
+__device__ __forceinline__ uint32_t pack2_e4m3(float a, float b, uint32_t old) {
+    const float ca = __builtin_fminf(__builtin_fmaxf(a, -448.0f), 448.0f), cb = __builtin_fminf(__builtin_fmaxf(b, -448.0f), 448.0f);
+    return (uint32_t)__builtin_amdgcn_cvt_pk_fp8_f32(a != a ? a : ca, b != b ? b : cb, (int)old, HIGH_HALF);
+}
+
+// fp8 store of a wave's 128 x 128 part of a tile held as 8 x 8 accumulator blocks of 16 x 16 (lane l:
+// row l%16, columns 4(l/16) .. +3 of a block): per 16-row slab a lane's four values of a block become
+// one word of a per-wave LDS patch [16][128 + 16] bytes (the pad keeps the 64 word stores of a block on
+// 64 banks), and the slab leaves as 16-byte chunks of whole 128-byte rows.  `dst`: the wave's first
+// row and column; ld in bytes.
+__device__ __forceinline__ void store_tile_fp8_blocks(const f32x4 (&acc16)[2 * TM][2 * TN], unsigned char* smem, uint8_t* dst, int64_t ld,
+                                                      int lane, int wave) {
+    constexpr int COLS = 2 * TN * 16, LD = COLS + 16, CPR = COLS / 16;
+    static_assert(16 * CPR == 128, "two chunks per lane and slab");
+    unsigned char* patch = smem + wave * 4096;
+#pragma unroll
+    for (int i = 0; i < 2 * TM; ++i) {
+#pragma unroll
+        for (int j = 0; j < 2 * TN; ++j) {
+            // (pinned here: copies the compiler may hoist would keep all blocks' values alive at once)
+            float x0, x1, x2, x3;
+            asm volatile("v_accvgpr_read_b32 %0, %2\n\tv_accvgpr_read_b32 %1, %3" : "=&v"(x0), "=&v"(x1) : "a"(acc16[i][j][0]), "a"(acc16[i][j][1]));
+            asm volatile("v_accvgpr_read_b32 %0, %2\n\tv_accvgpr_read_b32 %1, %3" : "=&v"(x2), "=&v"(x3) : "a"(acc16[i][j][2]), "a"(acc16[i][j][3]));
+            const uint32_t w = pack2_e4m3<true>(x2, x3, pack2_e4m3<false>(x0, x1, 0u));
+            *(uint32_t*)(patch + (lane & 15) * LD + 16 * j + 4 * (lane >> 4)) = w;
+        }
+        asm volatile("" ::: "memory");   // the reads below see the stores above (different types, same bytes)
+#pragma unroll
+        for (int it = 0; it < 2; ++it) {
+            const int idx = it * 64 + lane, r = idx / CPR, c = idx % CPR;
+            const u32x4 v = *(const u32x4*)(patch + r * LD + c * 16);
+            st_stream((u32x4*)(dst + (int64_t)(16 * i + r) * ld + c * 16), v);
+        }
+        asm volatile("" ::: "memory");   // the next slab's stores stay behind these reads
+    }
+}
+
 // One workgroup tile.  PEERS_FIRST picks the order of the two accumulation phases (peers'
 // partial sums, k loop) for tiles whose peers are added on the matrix cores.
 // SPLIT: the workgroup is one of g.k_splits that share a tile of the last partial round: it
@@ -108,9 +149,13 @@ __device__ __forceinline__ void store_tile_bf16_blocks(const f32x4 (&acc16)[2 * 
 // partial last round of compute units while 224-column tiles fill whole rounds (8192 x 3584: 448
 // tiles = 1.75 rounds against 512 = 2).  Per flop the narrower tile reads 7 % more of A from LDS
 // and L2, which two full rounds more than pay for.
-template <bool B_NT, bool PEERS_FIRST, bool SPLIT = false, bool RAGGED = false, bool MI16 = false, int NB = 2 * TN>
+template <bool B_NT, bool PEERS_FIRST, bool SPLIT = false, bool RAGGED = false, bool MI16 = false, int NB = 2 * TN, bool F8 = false>
 __device__ __forceinline__ void gemm_dtl_tile(const GemmArgs& g, unsigned char* smem) {
     static_assert(NB == 2 * TN || (NB == 7 && MI16 && B_NT && !SPLIT && !RAGGED && !PEERS_FIRST), "224-column tile: plain NT products only");
+    // F8: the operands are fp8 (e4m3fn) and g describes them as bf16 matrices of half the width (g.K, g.lda, g.ldb in
+    // two-byte units), so a stage still holds 128-byte rows -- 128 k now -- and every load and LDS address below is unchanged;
+    // only the k-step differs (k_step8: 16x16x128 MFMAs on the same 16 x 16 accumulator blocks).
+    static_assert(!F8 || (MI16 && B_NT && !SPLIT && !RAGGED && !PEERS_FIRST && NB == 2 * TN), "fp8: plain NT products on whole tiles");
     constexpr int BNX = WN * NB * 16;                            // columns of the workgroup tile
     constexpr int WTNX = NB * 16;                                // columns of a wave
     constexpr int LOADS_B = BNX * BKD * 2 / 1024 / (WM * WN);    // LDS-DMA loads of B per wave per k-step: 8 or 7
@@ -309,6 +354,42 @@ __device__ __forceinline__ void gemm_dtl_tile(const GemmArgs& g, unsigned char* 
             const s16x8 v = {lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
             bfr16[buf][bj] = __builtin_bit_cast(bf16x8, v);
         }
+    };
+
+    // fp8, 16x16x128 blocks: lane -> row (lane & 15) of a 16-row block and the 32 k at pieces 2q, 2q+1 (q = lane >> 4) of the
+    // row's eight -- two 16-byte reads, the halves of the operand's eight registers.  Both operands hand the matrix cores
+    // their k in this same order, which is all the sum needs.
+    typedef int i32x4 __attribute__((ext_vector_type(4)));
+    typedef int i32x8 __attribute__((ext_vector_type(8)));
+    typedef const __attribute__((address_space(3))) i32x4* lds_i32x4;
+    uint32_t fa8[2], fb8[2];
+    i32x8 af8[2][TM], bf8[2][2 * TN];   // A: blocks 0..3 and 4..7 of the current step; B: all blocks, this step's and the next one's
+    if constexpr (F8) {
+        const int p = lane & 15, gq = lane >> 4;
+        const int sw8 = (p >> 1) & 7;
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            fa8[h] = (uint32_t)((wm * WTM + p) * 128 + (((2 * gq + h) ^ sw8) << 4));
+            fb8[h] = B_BASE + (uint32_t)((wn * WTN + p) * 128 + (((2 * gq + h) ^ sw8) << 4));
+        }
+    }
+    // half h of fragment r of a stage: r = 0, 1: A block 0; 2 .. 17: B blocks 0 .. 7; 18 .. 23: A blocks 1 .. 3 (the order the
+    // first MFMAs of a step need them in); A blocks 4 .. 7 are read_a8_late
+    auto read_frag8 = [&](int buf, int r, uint32_t stage_off) __attribute__((always_inline)) {
+        const int h = r & 1;
+        if (r < 2 || r >= 18) {
+            const int bi = r < 2 ? 0 : (r - 16) / 2;
+            const i32x4 v = *(lds_i32x4)(size_t)(fa8[h] + stage_off + bi * 2048);
+            if (h == 0) af8[0][bi].lo = v; else af8[0][bi].hi = v;
+        } else {
+            const int bj = (r - 2) / 2;
+            const i32x4 v = *(lds_i32x4)(size_t)(fb8[h] + stage_off + bj * 2048);
+            if (h == 0) bf8[buf][bj].lo = v; else bf8[buf][bj].hi = v;
+        }
+    };
+    auto read_a8_late = [&](int r, uint32_t stage_off) __attribute__((always_inline)) {   // r = 0 .. 7: halves of A blocks 4 .. 7
+        const i32x4 v = *(lds_i32x4)(size_t)(fa8[r & 1] + stage_off + (4 + r / 2) * 2048);
+        if ((r & 1) == 0) af8[1][r / 2].lo = v; else af8[1][r / 2].hi = v;
     };
 
     // The accumulators start at the bias instead of zero when the whole tile lies in the reduce
@@ -580,11 +661,14 @@ __device__ __forceinline__ void gemm_dtl_tile(const GemmArgs& g, unsigned char* 
 #pragma unroll
     for (int q = 0; q < LOADS_TILE; ++q) issue_load(0, 0, q);
 #pragma unroll
-    for (int q = 0; q < kEarly; ++q) issue_load(1, 1, q);
-    __builtin_amdgcn_s_waitcnt(vmcnt_imm(kEarly));
+    for (int q = 0; q < (F8 ? LOADS_TILE : kEarly); ++q) issue_load(1, 1, q);   // (fp8: a step requests the whole next-but-one step)
+    __builtin_amdgcn_s_waitcnt(vmcnt_imm(F8 ? LOADS_TILE : kEarly));
     __builtin_amdgcn_s_barrier();
     KR_SCHED_FENCE();
-    if constexpr (MI16) {   // (A blocks 4..7 are read inside the first sub-step)
+    if constexpr (F8) {
+#pragma unroll
+        for (int r = 0; r < 24; ++r) read_frag8(0, r, 0);
+    } else if constexpr (MI16) {   // (A blocks 4..7 are read inside the first sub-step)
 #pragma unroll
         for (int j = 0; j < NB; ++j) read_b16(0, j, 0, 0);
 #pragma unroll
@@ -708,11 +792,66 @@ __device__ __forceinline__ void gemm_dtl_tile(const GemmArgs& g, unsigned char* 
             }
         }
     };
+    // The k-step on fp8 operands: 64 MFMAs of 16x16x128 (32 cycles each), rows of blocks in order; a step's B fragments live
+    // through the whole step, so B is double-buffered in registers (8 blocks x 8 registers x 2) and A in two halves of
+    // four blocks.
+    //   slots 0..7: A blocks 4..7 of this step (needed from slot 32 on);
+    //   behind slot kBarA8: every LDS read of the stage has returned -- barrier (a): the stage is free, and all 16 loads of
+    //     step t+2 go out, one per two MFMAs (64 cycles apart);
+    //   behind slot kBarB8: wait for the loads of step t+1 (the younger ones of step t+2 stay outstanding) -- barrier (b) --
+    //     and read all of B and A blocks 0..3 of step t+1: two reads per slot at first, then one.
+    constexpr int kBarA8 = 16, kBarB8 = 44;
+    constexpr int kLoadsBeforeB8 = (kBarB8 - kBarA8) / 2;   // loads of step t+2 in slots kBarA8+1, +3, ... <= kBarB8
+    static_assert(kLoadsBeforeB8 <= LOADS_PER_TILE && kBarA8 + 1 + 2 * (LOADS_PER_TILE - 1) < 64 && 10 + (63 - kBarB8 - 5) >= 24, "fp8 k-step schedule");
+    auto k_step8 = [&](int t, auto stage_c) __attribute__((always_inline)) {
+        const uint32_t stage_cur = stage_c;
+        const uint32_t stage_nxt = stage_cur ^ 1u;
+        const uint32_t st_cur = stage_cur * A_ST, st_nxt = stage_nxt * A_ST;
+        const int cur = stage_c, nxt = cur ^ 1;
+#pragma unroll
+        for (int s = 0; s < 64; ++s) {
+            const int i = s / 8, j = s % 8;
+            // (accumulator tied to its AGPRs, as in k_step16; formats left at their default, fp8 e4m3 for both operands)
+            asm volatile("v_mfma_f32_16x16x128_f8f6f4 %0, %1, %2, %0"
+                         : "+a"(acc16[i][j])
+                         : "v"(bf8[cur][j]), "v"(af8[i >> 2][i & 3]));
+            if (s < 8) read_a8_late(s, st_cur);
+            if (s == kBarA8) {
+                KR_SCHED_FENCE();
+                __builtin_amdgcn_s_waitcnt(kLgkm0);
+                __builtin_amdgcn_s_barrier();
+            }
+            if (s > kBarA8 && (s - kBarA8) % 2 == 1 && (s - kBarA8) / 2 < LOADS_PER_TILE) issue_load(t + 2, stage_cur, (s - kBarA8) / 2);
+            if (s == kBarB8) {
+                KR_SCHED_FENCE();
+                __builtin_amdgcn_s_waitcnt(vmcnt_imm(kLoadsBeforeB8));
+                __builtin_amdgcn_s_barrier();
+            }
+            if (s > kBarB8) {
+                const int u = s - kBarB8 - 1;   // 0 .. 18
+                if (u < 5) {
+                    read_frag8(nxt, 2 * u, st_nxt);
+                    read_frag8(nxt, 2 * u + 1, st_nxt);
+                } else if (10 + (u - 5) < 24) {
+                    read_frag8(nxt, 10 + (u - 5), st_nxt);
+                }
+            }
+            KR_SCHED_FENCE();
+        }
+    };
     // Main part: one trip = two k-steps, so every LDS stage offset is a compile-time constant
     // (immediate offsets on the fragment reads) and the loop branch is taken once per 128 MFMAs;
     // an odd last step follows.
     int t = 0;
-    if constexpr (MI16) {
+    if constexpr (F8) {
+#pragma nounroll
+        for (; t + 2 <= kt_total; t += 2) {
+            k_step8(t, std::integral_constant<uint32_t, 0>{});
+            k_step8(t + 1, std::integral_constant<uint32_t, 1>{});
+        }
+        pin_accumulators();
+        if (t < kt_total) k_step8(t, std::integral_constant<uint32_t, 0>{});
+    } else if constexpr (MI16) {
 #pragma nounroll
         for (; t + 2 <= kt_total; t += 2) {
             k_step16(t, std::integral_constant<uint32_t, 0>{});
@@ -763,7 +902,10 @@ __device__ __forceinline__ void gemm_dtl_tile(const GemmArgs& g, unsigned char* 
     }
     pin_accumulators();
     // peers and bias that are already in the accumulators are not added again
-    if constexpr (NB != 2 * TN) {
+    if (F8 && g.out_fp8) {
+        if constexpr (F8)
+            store_tile_fp8_blocks(acc16, smem, (uint8_t*)g.out + (int64_t)(m0 + wm * WTM) * g.N + n0 + wn * WTN, g.N, lane, wave);
+    } else if constexpr (NB != 2 * TN) {
         // 224-column tile of a plain product: every row goes to `out`
         store_tile_bf16_blocks<NB>(acc16, smem, (uint16_t*)g.out + (int64_t)(m0 + wm * WTM) * g.N + n0 + wn * WTNX, g.N, lane, wave);
     } else if constexpr (MI16) {
@@ -806,7 +948,21 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_dtl16n7_kernel(const GemmArg
     gemm_dtl_tile<true, false, false, false, true, 7>(g, smem);
 }
 
+// fp8 (e4m3fn) operands, transposed-contiguous B, whole 256 x 256 tiles; the result is fp8, bf16 or fp32.
+__global__ __launch_bounds__(WM* WN * 64) void gemm_dtl8_kernel(const GemmArgs g) {
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+    gemm_dtl_tile<true, false, false, false, true, 2 * TN, true>(g, smem);
+}
+
 }  // namespace
+
+// g as for the bf16 kernel with the fp8 operands described in two-byte units (K, lda, ldb halved).
+hipError_t launch_gemm_dtl8(const GemmArgs& g, hipStream_t st) {
+    static std::atomic<uint64_t> opted;
+    if (hipError_t e = lds_opt_in((const void*)gemm_dtl8_kernel, LDS_BYTES, opted); e != hipSuccess) return e;
+    hipLaunchKernelGGL(gemm_dtl8_kernel, dim3((unsigned)(g.tiles_m * g.tiles_n)), dim3(WM * WN * 64), LDS_BYTES, st, g);
+    return hipGetLastError();
+}
 
 // Second launch of a call with a split tail: g.k_splits workgroups per tile of the last partial
 // round (g.out = workspace).

@@ -39,7 +39,11 @@ def _matmul_w_progress(a, a_local, b, progress, configs, status=None) -> torch.T
 
 
 def _all_gather_matmul_fp8(peers: PeerBuffers, b, a_out, progress, **kwargs):
-    """The fp8 branch of ``all_gather_matmul``: convert, multiply in bf16 with an fp32 result, round once."""
+    """The fp8 branch of ``all_gather_matmul`` (``all_gather_matmul.py:53,121,213``): fp8 product with fp32
+    accumulation, rounded to fp8 once.  Shapes the fp8 kernel takes (M, N multiples of 256, K of 128) run on
+    the fp8 matrix-core instruction (``kr_gemm_fp8``); others are widened to bf16 (exact), multiplied by the
+    bf16 kernels with an fp32 result, and rounded by ``kr_cast_f32_to_fp8`` -- the same sums up to fp32
+    summation order.  ``fp8_kernel=False`` forces the widening path."""
     fp8 = torch.float8_e4m3fn
     W = peers.W
     m, K = peers.slice(0).shape
@@ -65,6 +69,11 @@ def _all_gather_matmul_fp8(peers: PeerBuffers, b, a_out, progress, **kwargs):
         a_out = a_full
     if progress is not None:
         progress.fill_(1)
+    if kwargs.get("fp8_kernel", True) and M % 256 == 0 and N % 256 == 0 and K % 128 == 0:
+        c = torch.empty((M, N), dtype=fp8, device=dev)
+        _lib.check(lib.kr_gemm_fp8(a_full.data_ptr(), K, b.T.data_ptr(), K, M, N, K, c.data_ptr(), 2, stream),
+                   "all_gather_matmul(fp8)")
+        return a_out, c
     a16 = torch.empty((M, K), dtype=torch.bfloat16, device=dev)
     bt16 = torch.empty((N, K), dtype=torch.bfloat16, device=dev)           # b.T is contiguous: memory [N, K]
     _lib.check(lib.kr_cast_fp8_to_bf16(a_full.data_ptr(), M * K, a16.data_ptr(), stream), "cast_fp8_to_bf16(a)")

@@ -353,6 +353,26 @@ def test_fp8_cast_argument_errors(lib):
         assert f(None, 0, None, None) == 0
 
 
+def test_gemm_fp8_argument_errors(lib):
+    f = lib.kr_gemm_fp8
+    ok = (FAKE, 512, FAKE, 512, 256, 256, 512, FAKE, 2, None)
+    def call(**kw):
+        names = ("A", "lda", "Bt", "ldb", "M", "N", "K", "out", "kind", "stream")
+        args = dict(zip(names, ok)); args.update(kw)
+        return f(*[args[n] for n in names])
+    assert call(M=128) == _lib.KR_ERR_BAD_DIM            # whole 256 x 256 tiles only
+    assert call(N=384) == _lib.KR_ERR_BAD_DIM
+    assert call(K=192, lda=192, ldb=192) == _lib.KR_ERR_BAD_DIM
+    assert call(kind=3) == _lib.KR_ERR_BAD_DIM
+    assert call(M=-256) == _lib.KR_ERR_BAD_DIM
+    assert call(A=None) == _lib.KR_ERR_NULL_POINTER
+    assert call(out=None) == _lib.KR_ERR_NULL_POINTER
+    assert call(lda=256) == _lib.KR_ERR_LAYOUT           # rows shorter than K
+    assert call(ldb=520) == _lib.KR_ERR_ALIGNMENT        # row stride not a multiple of 16 bytes
+    assert call(Bt=FAKE + 8) == _lib.KR_ERR_ALIGNMENT
+    assert call(M=0, A=None, Bt=None, out=None) == 0     # nothing to do, nothing launched
+
+
 def test_probe_argument_errors(lib):
     assert lib.kr_probe_read(FAKE, 24, None, None) == _lib.KR_ERR_NUMEL_MOD8
     assert lib.kr_probe_read(None, 32, None, None) == _lib.KR_ERR_NULL_POINTER

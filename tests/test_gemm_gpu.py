@@ -155,6 +155,70 @@ def test_all_gather_matmul_fp8(dev):
         fused.all_gather_matmul(a.to(dev), bT.to(dev).T, gather=True)
 
 
+@pytest.mark.parametrize("K", [128, 256, 384, 1024])
+def test_fp8_kernel_exact_sums(dev, K):
+    """kr_gemm_fp8 (fp8 operands on the fp8 matrix-core instruction): with small integers and halves every
+    fp32 sum is exact whatever its order, so all three result types equal the oracle bit for bit -- the fp8
+    result with its saturated elements, through the wrapper and straight through the C ABI; one, two, an odd
+    number and many k-steps."""
+    fp8 = torch.float8_e4m3fn
+    W, m, N = 8, 64, 768
+    g = torch.Generator().manual_seed(31 + K)
+    a = torch.randint(-2, 3, (W, m, K), generator=g).float().to(fp8)
+    bT = (torch.randint(-3, 4, (N, K), generator=g).float() * 0.5).to(fp8)
+    a[0], a[1], bT[:64] = 4.0, -4.0, 1.5            # sums of +-6K: beyond the largest fp8 value on both sides
+    a_full, want = orc.all_gather_matmul_fp8(a, bT.T)
+    exact = a.reshape(W * m, K).float() @ bT.float().T
+    assert (exact > 448).any() and (exact < -448).any() and (exact.abs() < 448).any()      # the case has saturating and ordinary sums
+    a_out, c = fused.all_gather_matmul(a.to(dev), bT.to(dev).T, rank=2)
+    assert c.dtype == fp8 and torch.equal(a_out.cpu().view(torch.uint8), a_full.view(torch.uint8))
+    assert torch.equal(c.cpu().view(torch.uint8), want.view(torch.uint8))
+    lib = _lib.load()
+    stream = torch.cuda.current_stream(dev).cuda_stream
+    ad, bd = a.reshape(W * m, K).to(dev), bT.to(dev)
+    for kind, dtype in ((1, torch.float32), (0, BF16)):
+        out = torch.full((W * m, N), 7, dtype=dtype, device=dev)
+        assert lib.kr_gemm_fp8(ad.data_ptr(), K, bd.data_ptr(), K, W * m, N, K, out.data_ptr(), kind, stream) == 0
+        assert torch.equal(out.cpu(), exact.to(dtype))
+
+
+def test_fp8_kernel_random_operands_and_nan(dev):
+    """Random operands: within one fp8 step of the oracle and of the widening path (the orders of the fp32
+    sums differ), mostly equal; the fp32 result against a double-precision product; row strides larger than
+    K; a NaN operand element makes its row of the result NaN and nothing else."""
+    fp8 = torch.float8_e4m3fn
+    W, m, K, N = 8, 128, 2048, 1280
+    g = torch.Generator().manual_seed(41)
+    a = torch.randn(W, m, K, generator=g).to(fp8)
+    bT = (torch.randn(N, K, generator=g) * 0.05).to(fp8)
+    _, c = fused.all_gather_matmul(a.to(dev), bT.to(dev).T)
+    _, c_wide = fused.all_gather_matmul(a.to(dev), bT.to(dev).T, fp8_kernel=False)
+    _, want = orc.all_gather_matmul_fp8(a, bT.T)
+    ref = want.float()
+    step = torch.maximum(ref.abs(), torch.tensor(2.0 ** -6)) * 2.0 ** -3          # spacing of e4m3 at that magnitude
+    for got in (c.cpu().float(), c_wide.cpu().float()):
+        assert (got == ref).float().mean() > 0.99
+        assert ((got - ref).abs() <= step).all()
+    lib = _lib.load()
+    stream = torch.cuda.current_stream(dev).cuda_stream
+    M = W * m
+    a_pad = torch.zeros(M, K + 64, dtype=torch.uint8).view(fp8)
+    a_pad[:, :K] = a.reshape(M, K)
+    b_pad = torch.zeros(N, K + 16, dtype=torch.uint8).view(fp8)
+    b_pad[:, :K] = bT
+    ad, bd = a_pad.to(dev), b_pad.to(dev)
+    out = torch.empty(M, N, dtype=torch.float32, device=dev)
+    assert lib.kr_gemm_fp8(ad.data_ptr(), K + 64, bd.data_ptr(), K + 16, M, N, K, out.data_ptr(), 1, stream) == 0
+    exact = (a.reshape(M, K).double() @ bT.double().T)
+    torch.testing.assert_close(out.cpu().double(), exact, rtol=1e-5, atol=1e-3)      # fp32 sums of 2048 products of size 0.05
+    a_nan = a.reshape(M, K).clone()
+    a_nan.view(torch.uint8)[300, 77] = 0x7f
+    c = torch.empty(M, N, dtype=fp8, device=dev)
+    assert lib.kr_gemm_fp8(a_nan.to(dev).data_ptr(), K, bT.to(dev).data_ptr(), K, M, N, K, c.data_ptr(), 2, stream) == 0
+    nan = torch.isnan(c.cpu().float())
+    assert nan[300].all() and not nan[:300].any() and not nan[301:].any()
+
+
 def test_split_fp32_is_one_pass_and_bit_exact(dev):
     """kr_split_fp32 writes the hi / lo blocks of an fp32 operand in the three layouts the GEMM
     wrappers use, bit for bit what elementwise torch ops give (hi = bf16(x), lo = bf16(x - hi)),
