@@ -646,23 +646,28 @@ __device__ __forceinline__ void gemm_dtl_tile(const GemmArgs& g, unsigned char* 
     pin_accumulators();
 
     // ---- prologue: request k-step 0 and the first loads of step 1; wait for step 0 ------------
-    // How the LOADS_PER_TILE loads of a k-step are spread: kEarly go out right behind the barrier
-    // that frees their stage (rest of sub-step 3 of step t-2), the others during sub-steps 0 and
+    // How the LOADS_PER_TILE loads of a k-step are spread.  32x32x16 form: kEarly go out right behind the
+    // barrier that frees their stage (rest of sub-step 3 of step t-2), the others during sub-steps 0 and
     // 1 of step t-1 -- every second MFMA.  One per MFMA from four waves is twice what the CU's
-    // address unit takes (the waves then stall at issue); spreading them evenly over the whole
-    // step leaves the last ones too little time before the barrier that needs them.
-    // (16x16x32 form: its MFMAs are half as long, so a load issued during the step that needs it
-    // has half as many MFMAs to hide behind; there 14 loads of step t+2 go out behind the barrier
-    // of step t, one per four MFMAs -- 64 cycles apart, as above -- and the last two at the start
-    // of step t+1)
-    // (224-column tile: 15 loads per k-step and 56 MFMAs per sub-step: 12 behind the barrier, 3 at the start)
-    constexpr int kEarly = MI16 ? (NB == 7 ? 12 : 14) : 6;
-    static_assert(NSTAGE == 2 && LOADS_PER_TILE == 16 && (LOADS_TILE == 16 || (NB == 7 && LOADS_TILE == 15)), "load schedule below: 6 + 8 + 2 loads");
+    // address unit takes (the waves then stall at issue).
+    // 16x16x32 form: the stage is free early in the step (barrier (a) of k_step16, behind slot kBarA0 of
+    // sub-step 0), and from there the loads of step t+2 go out evenly over a whole step's worth of
+    // slots -- one per eight MFMAs (seven in the 224-column tile), 128 cycles apart; those that fall
+    // behind the end of step t are the first thing step t+1 issues (kInStep counts the others).
+    // fp8 form: see k_step8.
+    constexpr int kEarly = 6;
+    constexpr int kFrags16 = NB + 2 * TM;                              // fragments of a sub-step: 16 or 15
+    constexpr int kBarA0 = 2 * (kFrags16 - 1) + (NB == 7 ? 8 : 10);    // slot of sub-step 0 behind which every read of the stage has returned
+    constexpr int kLoadGap16 = NB == 7 ? 7 : 8;
+    constexpr int kSlots16 = 2 * 2 * TM * NB;                          // MFMAs of a k-step: 128 or 112
+    constexpr int kInStep = (kSlots16 - 1 - kBarA0 - 2) / kLoadGap16 + 1 < LOADS_TILE ? (kSlots16 - 1 - kBarA0 - 2) / kLoadGap16 + 1 : LOADS_TILE;
+    constexpr int kFirst = F8 ? LOADS_TILE : MI16 ? kInStep : kEarly;   // loads of step 1 the prologue issues
+    static_assert(NSTAGE == 2 && LOADS_PER_TILE == 16 && (LOADS_TILE == 16 || (NB == 7 && LOADS_TILE == 15)), "load schedules below");
 #pragma unroll
     for (int q = 0; q < LOADS_TILE; ++q) issue_load(0, 0, q);
 #pragma unroll
-    for (int q = 0; q < (F8 ? LOADS_TILE : kEarly); ++q) issue_load(1, 1, q);   // (fp8: a step requests the whole next-but-one step)
-    __builtin_amdgcn_s_waitcnt(vmcnt_imm(F8 ? LOADS_TILE : kEarly));
+    for (int q = 0; q < kFirst; ++q) issue_load(1, 1, q);
+    __builtin_amdgcn_s_waitcnt(vmcnt_imm(kFirst));
     __builtin_amdgcn_s_barrier();
     KR_SCHED_FENCE();
     if constexpr (F8) {
@@ -727,27 +732,32 @@ __device__ __forceinline__ void gemm_dtl_tile(const GemmArgs& g, unsigned char* 
     // so fragment reads and loads get MFMA slots of their own.  Row i of MFMAs needs A block i and
     // all B blocks, so a sub-step can start on the B blocks and the first A blocks; the others
     // follow while it runs.
-    //   sub-step 0: the fragments of sub-step 1 (every fourth slot), A blocks 4..7 of this
-    //     sub-step (slots 1, 9, 17, 25), the last two loads of step t+1 (slots 2, 6);
-    //   sub-step 1, behind MFMA 7: every LDS read of the stage has returned -- barrier (a): the
-    //     stage is free, the loads of step t+2 start (one per four MFMAs);
-    //   behind MFMA 47: wait for the loads of step t+1 (the ten younger ones of step t+2 stay
-    //     outstanding) -- barrier (b) -- and read the B blocks and A blocks 0..3 of step t+1.
-    // Two barriers instead of one buy the loads a third more time to arrive (from slot 9 of one
-    // step to slot 47 of the next): the wait sits right in front of the first read that needs
-    // the data, not in front of the first load that needs the room.
-    // (224-column tile, NB = 7: 56 MFMAs per sub-step; everything keeps its distance from the end of
-    // the sub-step: barrier (a) behind MFMA 6, barrier (b) behind MFMA 39, the same 16 slots behind it
-    // for the 7 + 4 fragments of the next step; 15 fragments of sub-step 1 to read in sub-step 0)
+    //   sub-step 0: the fragments of sub-step 1 (every second slot), A blocks 4..7 of this
+    //     sub-step (slots 1, 9, 17, 25), the last loads of step t+1;
+    //   behind slot kBarA0 of sub-step 0: every LDS read of the stage has returned -- barrier (a):
+    //     the stage is free, the loads of step t+2 start (one per eight MFMAs, through the rest of
+    //     the step);
+    //   sub-step 1, behind MFMA 47: wait for the loads of step t+1 (the younger ones of step t+2
+    //     stay outstanding) -- barrier (b) -- and read the B blocks and A blocks 0..3 of step t+1.
+    // The wait sits right in front of the first read that needs the data, not in front of the first
+    // load that needs the room.  Reading sub-step 1's fragments in the first half of sub-step 0 (they
+    // used to take all of it, with barrier (a) in sub-step 1 and the loads crowded into what was left
+    // of the step, 64 cycles apart) is what makes room for the even spacing: same process, rotating
+    // operands, 8192x8192x3584 row-major B with its band 356-357 -> 348-349 us, 8192x3584x8192
+    // transposed B on 224-column tiles 326-327 -> 325-326 us, 4096x8192x1024 with seven peers
+    // 118.2 -> 117.2 us; with the early barrier alone and the loads still 64 cycles apart nothing moves.
+    // (224-column tile, NB = 7: 56 MFMAs per sub-step; barrier (b) behind MFMA 39, the same 16 slots
+    // behind it for the 7 + 4 fragments of the next step; 15 fragments of sub-step 1 to read in sub-step 0)
     constexpr int NM16 = 2 * TM * NB;
     auto read_frag16 = [&](int buf, int r, int ks2, uint32_t stage_off) __attribute__((always_inline)) {
         if (r < NB) read_b16(buf, r, ks2, stage_off);
         else read_a16(buf, r - NB, ks2, stage_off);
     };
-    constexpr int kBarA = NB - 1;          // last MFMA of the first row
     constexpr int kBarB = NM16 - 17;
-    constexpr int kLoadsBeforeB = (kBarB - kBarA - 2) / 4 + 1;   // loads of step t+2 in slots 9, 13, ... < kBarB
-    static_assert(!MI16 || ((kLoadsBeforeB == 10 || (NB == 7 && kLoadsBeforeB == 8)) && kLoadsBeforeB <= kEarly), "wait count of barrier (b)");
+    // loads of step t+2 issued before the wait of barrier (b) (slots kBarA0 + 2, + kLoadGap16, ... <= NM16 + kBarB)
+    constexpr int kLoadsBeforeB = (NM16 + kBarB - kBarA0 - 2) / kLoadGap16 + 1 < kInStep ? (NM16 + kBarB - kBarA0 - 2) / kLoadGap16 + 1 : kInStep;
+    static_assert(!MI16 || (kBarA0 < NM16 && kBarA0 + 2 + kLoadGap16 * (LOADS_TILE - 1) - kSlots16 < kBarA0 + 2),
+                  "a step's late loads go out before the next step's first ones");
     auto k_step16 = [&](int t, auto stage_c) __attribute__((always_inline)) {
         const uint32_t stage_cur = stage_c;
         const uint32_t stage_nxt = stage_cur ^ 1u;
@@ -764,20 +774,21 @@ __device__ __forceinline__ void gemm_dtl_tile(const GemmArgs& g, unsigned char* 
                 asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0"
                              : "+a"(acc16[i][j])
                              : "v"(bfr16[cur][j]), "v"(af16[cur][i]));
+                const int slot = ks2 * NM16 + s;               // slot of the step
+                const int lq = slot - kBarA0 - 2;              // loads of step t+2: slots kBarA0 + 2 + kLoadGap16 * q
+                const int lw = lq + kSlots16;                  // ... and those of step t+1 that fell behind the end of step t-1
                 if (ks2 == 0) {
-                    if (s % 4 == 0) read_frag16(nxt, s / 4, 1, st_cur);
-                    if (NB == 7 && s == NM16 - 3) read_frag16(nxt, NB + 2 * TM - 1, 1, st_cur);   // the fifteenth
+                    if (s % 2 == 0 && s / 2 < kFrags16) read_frag16(nxt, s / 2, 1, st_cur);
                     if (s % 8 == 1 && s / 8 + 4 < 2 * TM) read_a16(cur, s / 8 + 4, 0, st_cur);
-                    // the last loads of step t+1
-                    if (s % 4 == 2 && s < 16 && kEarly + s / 4 < LOADS_TILE) issue_load(t + 1, stage_nxt, kEarly + s / 4);
-                } else {
-                    if (s == kBarA) {
+                    if (s == kBarA0) {
                         KR_SCHED_FENCE();
                         __builtin_amdgcn_s_waitcnt(kLgkm0);
                         __builtin_amdgcn_s_barrier();
                     }
-                    if (s > kBarA && (s - kBarA - 1) % 4 == 1 && (s - kBarA - 1) / 4 < kEarly)
-                        issue_load(t + 2, stage_cur, (s - kBarA - 1) / 4);
+                }
+                if (lq >= 0 && lq % kLoadGap16 == 0 && lq / kLoadGap16 < kInStep) issue_load(t + 2, stage_cur, lq / kLoadGap16);
+                if (lw % kLoadGap16 == 0 && lw / kLoadGap16 >= kInStep && lw / kLoadGap16 < LOADS_TILE) issue_load(t + 1, stage_nxt, lw / kLoadGap16);
+                if (ks2 == 1) {
                     if (s == kBarB) {
                         KR_SCHED_FENCE();
                         __builtin_amdgcn_s_waitcnt(vmcnt_imm(kLoadsBeforeB));
@@ -796,13 +807,18 @@ __device__ __forceinline__ void gemm_dtl_tile(const GemmArgs& g, unsigned char* 
     // through the whole step, so B is double-buffered in registers (8 blocks x 8 registers x 2) and A in two halves of
     // four blocks.
     //   slots 0..7: A blocks 4..7 of this step (needed from slot 32 on);
-    //   behind slot kBarA8: every LDS read of the stage has returned -- barrier (a): the stage is free, and all 16 loads of
-    //     step t+2 go out, one per two MFMAs (64 cycles apart);
+    //   behind slot kBarA8: every LDS read of the stage has returned -- barrier (a): the stage is free, and the 16 loads of
+    //     step t+2 go out, one per three MFMAs (96 cycles apart: measured 3-5 % faster than 64 cycles apart);
     //   behind slot kBarB8: wait for the loads of step t+1 (the younger ones of step t+2 stay outstanding) -- barrier (b) --
-    //     and read all of B and A blocks 0..3 of step t+1: two reads per slot at first, then one.
-    constexpr int kBarA8 = 16, kBarB8 = 44;
-    constexpr int kLoadsBeforeB8 = (kBarB8 - kBarA8) / 2;   // loads of step t+2 in slots kBarA8+1, +3, ... <= kBarB8
-    static_assert(kLoadsBeforeB8 <= LOADS_PER_TILE && kBarA8 + 1 + 2 * (LOADS_PER_TILE - 1) < 64 && 10 + (63 - kBarB8 - 5) >= 24, "fp8 k-step schedule");
+    //     and read all of B and A blocks 0..3 of step t+1, one half-fragment per slot (two per slot at first, were the
+    //     barrier later than slot 39).
+    // Same-process comparison of (kBarA8, kBarB8, gap) on 8192x4096x8192, 4096x6656x16384, 8192x8192x3584, rotating operands:
+    // (16, 44, 2) 188 / 313-320 / 169-170 us, (16, 40, 2) 184 / 308-312 / 167, (16, 39, 3) 179 / 297-300 / 164-165,
+    // (12, 39, 3) 174-176 / 296-298 / 164 (hipBLASLt's scaled fp8 product in the same runs: 168-172 / 304-305 / 160-165).
+    constexpr int kBarA8 = 12, kBarB8 = 39, kLoadGap8 = 3;
+    constexpr int kLoadsBeforeB8 = (kBarB8 - kBarA8 - 1) / kLoadGap8 + 1 < LOADS_PER_TILE ? (kBarB8 - kBarA8 - 1) / kLoadGap8 + 1 : LOADS_PER_TILE;   // loads of step t+2 in slots <= kBarB8
+    constexpr int kReadSlots8 = 63 - kBarB8, kDoubleReads8 = kReadSlots8 < 24 ? 24 - kReadSlots8 : 0;   // 24 fragment halves behind barrier (b): two per slot at first
+    static_assert(kBarA8 >= 8 && kBarB8 > kBarA8 && kBarA8 + 1 + kLoadGap8 * (LOADS_PER_TILE - 1) < 64 && kDoubleReads8 <= kReadSlots8, "fp8 k-step schedule");
     auto k_step8 = [&](int t, auto stage_c) __attribute__((always_inline)) {
         const uint32_t stage_cur = stage_c;
         const uint32_t stage_nxt = stage_cur ^ 1u;
@@ -821,19 +837,20 @@ __device__ __forceinline__ void gemm_dtl_tile(const GemmArgs& g, unsigned char* 
                 __builtin_amdgcn_s_waitcnt(kLgkm0);
                 __builtin_amdgcn_s_barrier();
             }
-            if (s > kBarA8 && (s - kBarA8) % 2 == 1 && (s - kBarA8) / 2 < LOADS_PER_TILE) issue_load(t + 2, stage_cur, (s - kBarA8) / 2);
+            if (s > kBarA8 && (s - kBarA8 - 1) % kLoadGap8 == 0 && (s - kBarA8 - 1) / kLoadGap8 < LOADS_PER_TILE)
+                issue_load(t + 2, stage_cur, (s - kBarA8 - 1) / kLoadGap8);
             if (s == kBarB8) {
                 KR_SCHED_FENCE();
                 __builtin_amdgcn_s_waitcnt(vmcnt_imm(kLoadsBeforeB8));
                 __builtin_amdgcn_s_barrier();
             }
             if (s > kBarB8) {
-                const int u = s - kBarB8 - 1;   // 0 .. 18
-                if (u < 5) {
+                const int u = s - kBarB8 - 1;
+                if (u < kDoubleReads8) {
                     read_frag8(nxt, 2 * u, st_nxt);
                     read_frag8(nxt, 2 * u + 1, st_nxt);
-                } else if (10 + (u - 5) < 24) {
-                    read_frag8(nxt, 10 + (u - 5), st_nxt);
+                } else if (kDoubleReads8 + u < 24) {
+                    read_frag8(nxt, kDoubleReads8 + u, st_nxt);
                 }
             }
             KR_SCHED_FENCE();
