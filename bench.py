@@ -54,6 +54,7 @@ sys.path.insert(0, str(ROOT))
 
 HBM_PEAK_GBS = 8000.0            # MI355X HBM3E
 MFMA_BF16_PEAK_TFLOPS = 2500.0   # MI355X dense bf16
+MFMA_FP8_PEAK_TFLOPS = 5000.0    # MI355X dense fp8
 W = 8
 SETTLE_MS = 60.0                 # launches of the workload itself in front of every timed region
 GRAPH_REPLAYS = 15               # timed replays of a microsecond workload's graph
@@ -119,6 +120,8 @@ class Workload:
     cpu_repeats = 5
     use_graph = False      # microsecond kernels: time replays of a HIP graph of the launches
     has_vendor = False     # GEMMs: vendor_step() runs the vendor library's bare product
+    vendor_what = "torch.matmul (hipBLASLt) of the same A and B, product only"
+    mfma_peak = MFMA_BF16_PEAK_TFLOPS   # matrix-core peak of the workload's arithmetic type
 
     def setup(self, dev):   # allocate device inputs (several rotated sets)
         raise NotImplementedError
@@ -513,6 +516,62 @@ class AllGatherMatmul(Workload):
         return d
 
 
+class AllGatherMatmulFP8(AllGatherMatmul):
+    """The fp8 branch of the all-gather matmul (kraken/fused/all_gather_matmul.py:53,121,213) at the
+    reference's test shape: fp8 (e4m3fn) shards and weight, fp32 accumulation on the fp8 matrix-core
+    instruction, fp8 result.  Priced against the fp8 peak."""
+    dtype = "fp8 (e4m3fn) storage, fp32 accumulate"
+    mfma_peak = MFMA_FP8_PEAK_TFLOPS
+    vendor_what = "torch._scaled_mm (hipBLASLt) of the same fp8 A and B with unit scales, bf16 result"
+
+    def __init__(self, m=512, K=16384, N=6656, nsets=2):
+        super().__init__(m, K, N, nsets, False)
+        self.name = f"all_gather_matmul_fp8_{W * m}x{N}x{K}_w8"
+        self.bytes = W * m * K + K * N + W * m * N
+
+    def setup(self, dev):
+        import torch
+
+        fp8 = torch.float8_e4m3fn
+        g = torch.Generator().manual_seed(44)
+        self.hs = torch.randn(W, self.m, self.K, generator=g).to(fp8)
+        self.hbT = (torch.randn(self.N, self.K, generator=g) * 0.02).to(fp8)
+        gd = torch.Generator(device=dev).manual_seed(3)
+        self.s = [self.hs.to(dev)] + [torch.randn(W, self.m, self.K, generator=gd, device=dev).to(fp8) for _ in range(self.nsets - 1)]
+        self.bT = [self.hbT.to(dev)] + [(torch.randn(self.N, self.K, generator=gd, device=dev) * 0.02).to(fp8)
+                                        for _ in range(self.nsets - 1)]
+        self.c = [None] * self.nsets
+        self.one = torch.ones((), device=dev)
+
+    def vendor_step(self, i):
+        import torch
+
+        j = i % self.nsets
+        torch._scaled_mm(self.s[j].reshape(-1, self.K), self.bT[j].T, scale_a=self.one, scale_b=self.one, out_dtype=torch.bfloat16)
+
+    def check(self):
+        import torch
+        from oracle import oracle as orc
+
+        self.step(0)
+        rows = W * self.m
+        pick = torch.tensor([0, self.m - 1, 3 * self.m, rows - 1])
+        _, want = orc.all_gather_matmul_fp8(self.hs.reshape(-1, self.K)[pick].reshape(1, len(pick), self.K), self.hbT.T)
+        got, ref = self.c[0].cpu()[pick].float(), want.float()
+        step = torch.maximum(ref.abs(), torch.tensor(2.0 ** -6)) * 2.0 ** -3      # spacing of e4m3 at that magnitude
+        assert ((got - ref).abs() <= step).all() and (got == ref).float().mean() > 0.98, "fp8 result differs from the oracle"
+        return "sampled rows within one fp8 step of the oracle (the orders of the fp32 sums differ), over 98 % equal"
+
+    def cpu_step(self):
+        from oracle import oracle as orc
+
+        return orc.all_gather_matmul_fp8(self.hs, self.hbT.T)
+
+    def describe(self):
+        return {"W": W, "m": self.m, "K": self.K, "N": self.N, "b_layout": "b.T contiguous", "kernel": "gemm_dtl8_kernel",
+                "operand_sets": self.nsets, "mfma": "v_mfma_f32_16x16x128_f8f6f4", "peak_priced_against": "fp8 dense, 5.0 PFLOP/s"}
+
+
 class GemmReduceScatterCE(Workload):
     """Copy-engine reduce-scatter variant at the reference's test shape
     (test/test_gemm_reduce_scatter.py:93-111): producer GEMM with per-band flags, band copies,
@@ -596,6 +655,7 @@ def make_workloads():
         "ref_gemm_reduce_scatter_ce_persistent": GemmReduceScatterCE,
         "ref_all_gather_matmul": lambda: AllGatherMatmul(512, 16384, 6656, 2, False),
         "ref_all_gather_matmul_overlapped": lambda: AllGatherMatmul(512, 16384, 6656, 2, True),
+        "ref_all_gather_matmul_fp8": AllGatherMatmulFP8,
     }
 
 
@@ -808,6 +868,7 @@ def measure_gpu(wl, steps, warmup, dev, floors=False):
         "gbps": wl.bytes / (ev_ms * 1e-3) / 1e9,
         "hbm_frac": wl.bytes / (ev_ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
         "bound": wl.bound,
+        "dtype": wl.dtype,
         "timing": (f"hip graph of {timed // st['n']} launches, median of {st['n']} replays" if wl.use_graph
                    else f"eager launches, median of {st['n']} event intervals of {st['launches_per_interval']} launch(es)"),
         "algorithmic_bytes": wl.bytes,
@@ -817,13 +878,13 @@ def measure_gpu(wl, steps, warmup, dev, floors=False):
     }
     if wl.flops:
         rec["tflops"] = wl.flops / (ev_ms * 1e-3) / 1e12
-        rec["mfma_frac"] = rec["tflops"] / MFMA_BF16_PEAK_TFLOPS
+        rec["mfma_frac"] = rec["tflops"] / wl.mfma_peak
         rec["algorithmic_flops"] = wl.flops
     is_mfma = wl.bound == "mfma"
     rec["roofline"] = {
         "bound": wl.bound,
         "achieved": rec["tflops"] if is_mfma else rec["gbps"],
-        "peak": MFMA_BF16_PEAK_TFLOPS if is_mfma else HBM_PEAK_GBS,
+        "peak": wl.mfma_peak if is_mfma else HBM_PEAK_GBS,
         "unit": "TFLOP/s" if is_mfma else "GB/s",
         "frac": rec["mfma_frac"] if is_mfma else rec["hbm_frac"],
         "traffic": traffic[0],
@@ -833,10 +894,10 @@ def measure_gpu(wl, steps, warmup, dev, floors=False):
         # the vendor library's bare product of the same rotating operands (no peers, bias or band),
         # same protocol, same run
         _, vst, _ = time_gpu_eager(wl.vendor_step, max(steps, MIN_EAGER_STEPS), warmup)
-        rec["vendor"] = {"what": "torch.matmul (hipBLASLt) of the same A and B, product only",
+        rec["vendor"] = {"what": wl.vendor_what,
                          "ms": vst["median_ms"], "min_ms": vst["min_ms"], "max_ms": vst["max_ms"],
                          "tflops": wl.flops / (vst["median_ms"] * 1e-3) / 1e12,
-                         "mfma_frac": wl.flops / (vst["median_ms"] * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS}
+                         "mfma_frac": wl.flops / (vst["median_ms"] * 1e-3) / 1e12 / wl.mfma_peak}
     if floors and wl.use_graph and hasattr(wl, "floor_src"):
         rec["floors_us"] = floors_of(wl, steps, warmup)
     wl.release()
@@ -952,7 +1013,8 @@ def main() -> None:
     is_mfma = main_wl.bound == "mfma"
     value = rec["tflops"] if is_mfma else rec["gbps"]
     line = {
-        "metric": "bf16 TFLOP/s, GEMM + reduce epilogue" if is_mfma else "HBM GB/s, W-way reduce (algorithmic bytes / time)",
+        "metric": (("fp8" if main_wl.mfma_peak == MFMA_FP8_PEAK_TFLOPS else "bf16") + " TFLOP/s, GEMM + reduce epilogue") if is_mfma
+                  else "HBM GB/s, W-way reduce (algorithmic bytes / time)",
         "value": value,
         "unit": "TFLOP/s" if is_mfma else "GB/s",
         "n_gpus": 1,
@@ -963,7 +1025,7 @@ def main() -> None:
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
-        "dtype": "bf16",
+        "dtype": "fp8" if is_mfma and main_wl.mfma_peak == MFMA_FP8_PEAK_TFLOPS else "bf16",
         "data": "synthetic",
         "config": {"workload": main_wl.name, **main_wl.describe()},
         "parity": rec["parity"],

@@ -661,7 +661,9 @@ __device__ __forceinline__ void gemm_dtl_tile(const GemmArgs& g, unsigned char* 
     constexpr int kLoadGap16 = NB == 7 ? 7 : 8;
     constexpr int kSlots16 = 2 * 2 * TM * NB;                          // MFMAs of a k-step: 128 or 112
     constexpr int kInStep = (kSlots16 - 1 - kBarA0 - 2) / kLoadGap16 + 1 < LOADS_TILE ? (kSlots16 - 1 - kBarA0 - 2) / kLoadGap16 + 1 : LOADS_TILE;
-    constexpr int kFirst = F8 ? LOADS_TILE : MI16 ? kInStep : kEarly;   // loads of step 1 the prologue issues
+    constexpr int kBarA8 = 12, kBarB8 = 39, kLoadGap8 = 3;               // fp8 form (k_step8): barrier slots, slots between loads
+    constexpr int kInStep8 = (63 - kBarA8 - 1) / kLoadGap8 + 1 < LOADS_TILE ? (63 - kBarA8 - 1) / kLoadGap8 + 1 : LOADS_TILE;
+    constexpr int kFirst = F8 ? kInStep8 : MI16 ? kInStep : kEarly;   // loads of step 1 the prologue issues
     static_assert(NSTAGE == 2 && LOADS_PER_TILE == 16 && (LOADS_TILE == 16 || (NB == 7 && LOADS_TILE == 15)), "load schedules below");
 #pragma unroll
     for (int q = 0; q < LOADS_TILE; ++q) issue_load(0, 0, q);
@@ -814,11 +816,11 @@ __device__ __forceinline__ void gemm_dtl_tile(const GemmArgs& g, unsigned char* 
     //     barrier later than slot 39).
     // Same-process comparison of (kBarA8, kBarB8, gap) on 8192x4096x8192, 4096x6656x16384, 8192x8192x3584, rotating operands:
     // (16, 44, 2) 188 / 313-320 / 169-170 us, (16, 40, 2) 184 / 308-312 / 167, (16, 39, 3) 179 / 297-300 / 164-165,
-    // (12, 39, 3) 174-176 / 296-298 / 164 (hipBLASLt's scaled fp8 product in the same runs: 168-172 / 304-305 / 160-165).
-    constexpr int kBarA8 = 12, kBarB8 = 39, kLoadGap8 = 3;
-    constexpr int kLoadsBeforeB8 = (kBarB8 - kBarA8 - 1) / kLoadGap8 + 1 < LOADS_PER_TILE ? (kBarB8 - kBarA8 - 1) / kLoadGap8 + 1 : LOADS_PER_TILE;   // loads of step t+2 in slots <= kBarB8
+    // (12, 39, 3) 174-176 / 296-298 / 164 (hipBLASLt's scaled fp8 product in the same runs: 168-172 / 304-305 / 160-165);
+    // (12, 39, 4) and (12, 43, 4), whose last loads go out at the start of the next step, measure like (12, 39, 3).
+    constexpr int kLoadsBeforeB8 = (kBarB8 - kBarA8 - 1) / kLoadGap8 + 1 < kInStep8 ? (kBarB8 - kBarA8 - 1) / kLoadGap8 + 1 : kInStep8;   // loads of step t+2 in slots <= kBarB8
     constexpr int kReadSlots8 = 63 - kBarB8, kDoubleReads8 = kReadSlots8 < 24 ? 24 - kReadSlots8 : 0;   // 24 fragment halves behind barrier (b): two per slot at first
-    static_assert(kBarA8 >= 8 && kBarB8 > kBarA8 && kBarA8 + 1 + kLoadGap8 * (LOADS_PER_TILE - 1) < 64 && kDoubleReads8 <= kReadSlots8, "fp8 k-step schedule");
+    static_assert(kBarA8 >= 8 && kBarB8 > kBarA8 && kBarA8 + 1 + kLoadGap8 * (LOADS_PER_TILE - 1) - 64 < kBarA8 + 1 && kDoubleReads8 <= kReadSlots8, "fp8 k-step schedule");
     auto k_step8 = [&](int t, auto stage_c) __attribute__((always_inline)) {
         const uint32_t stage_cur = stage_c;
         const uint32_t stage_nxt = stage_cur ^ 1u;
@@ -837,8 +839,10 @@ __device__ __forceinline__ void gemm_dtl_tile(const GemmArgs& g, unsigned char* 
                 __builtin_amdgcn_s_waitcnt(kLgkm0);
                 __builtin_amdgcn_s_barrier();
             }
-            if (s > kBarA8 && (s - kBarA8 - 1) % kLoadGap8 == 0 && (s - kBarA8 - 1) / kLoadGap8 < LOADS_PER_TILE)
+            if (s > kBarA8 && (s - kBarA8 - 1) % kLoadGap8 == 0 && (s - kBarA8 - 1) / kLoadGap8 < kInStep8)
                 issue_load(t + 2, stage_cur, (s - kBarA8 - 1) / kLoadGap8);
+            if ((s + 64 - kBarA8 - 1) % kLoadGap8 == 0 && (s + 64 - kBarA8 - 1) / kLoadGap8 >= kInStep8 && (s + 64 - kBarA8 - 1) / kLoadGap8 < LOADS_PER_TILE)
+                issue_load(t + 1, stage_nxt, (s + 64 - kBarA8 - 1) / kLoadGap8);   // the loads of step t+1 that fell behind the end of step t-1
             if (s == kBarB8) {
                 KR_SCHED_FENCE();
                 __builtin_amdgcn_s_waitcnt(vmcnt_imm(kLoadsBeforeB8));
