@@ -74,10 +74,11 @@ MEASURED_TRAFFIC = {
     "reduce_bias_rmsnorm_w8_16384x4096_large": (1208007579, "8eb5098"), # profiles/reduce_rmsnorm_kernel_w8_16384x4096.md
     # the GEMMs: L2 fills (A and B panels re-read per tile row / column, served mostly by the 256 MB
     # last-level cache, not by HBM) + write-backs
-    "gemm_reduce_scatter_8192x8192x3584_w8": (985115063, "d4fb59f"),    # profiles/gemm_dtl16_kernel_reduce_scatter_8192x8192x3584.md
-    "gemm_all_reduce_4096x8192x1024_w8": (707964399, "d4fb59f"),        # profiles/gemm_dtl16_kernel_all_reduce_4096x8192x1024.md
-    "all_gather_matmul_8192x3584x8192_w8": (836807009, "d4fb59f"),      # profiles/gemm_dtl16n7_kernel_all_gather_matmul_8192x3584x8192.md
-    "all_gather_matmul_4096x6656x16384_w8": (1853258856, "d4fb59f"),    # profiles/gemm_dtl16_kernel_all_gather_matmul_4096x6656x16384.md
+    "gemm_reduce_scatter_8192x8192x3584_w8": (986499754, "ffe923e"),    # profiles/gemm_dtl16_kernel_reduce_scatter_8192x8192x3584.md
+    "gemm_all_reduce_4096x8192x1024_w8": (708047563, "ffe923e"),        # profiles/gemm_dtl16_kernel_all_reduce_4096x8192x1024.md
+    "all_gather_matmul_8192x3584x8192_w8": (837421610, "ffe923e"),      # profiles/gemm_dtl16n7_kernel_all_gather_matmul_8192x3584x8192.md
+    "all_gather_matmul_4096x6656x16384_w8": (1894179528, "ffe923e"),    # profiles/gemm_dtl16_kernel_all_gather_matmul_4096x6656x16384.md
+    "all_gather_matmul_fp8_4096x6656x16384_w8": (851641889, "ffe923e"),  # profiles/gemm_dtl8_kernel_all_gather_matmul_fp8_4096x6656x16384.md
 }
 
 # Targets of the benchmark definition: fraction of the binding roof.  The W = 8 reduce(+bias+RMSNorm)
