@@ -494,6 +494,19 @@ int kr_gemm_fp8(const void* A, int64_t lda, const void* Bt, int64_t ldb, int64_t
                 void* out, int out_kind, void* stream);
 
 /*
+ * kr_gemm_fp8 for an A whose rows arrive while the kernel runs -- the fp8 form of kr_all_gather_matmul_bf16
+ * (same flags, local shard, tile order, wait limit and status word; see there), which is what the reference's
+ * one kernel is when its shards are fp8 (kraken/fused/all_gather_matmul.py:25-123 with
+ * dtype = tl.float8e4nv, :53, :121, launched by _matmul_w_progress :147-219).
+ *   A, A_local: fp8, row strides lda, lda_local in bytes (multiples of 16); Bt, out, out_kind as for kr_gemm_fp8.
+ * M % 256 == 0, N % 256 == 0, K % 128 == 0, M % (W * splits_per_rank) == 0, 0 <= rank < W.
+ */
+int kr_all_gather_matmul_fp8(const void* A, int64_t lda, const void* A_local, int64_t lda_local, const void* Bt,
+                             int64_t ldb, int64_t M, int64_t N, int64_t K, int W, int rank, int splits_per_rank,
+                             const uint32_t* progress, int64_t wait_limit_us, int32_t* status, void* out, int out_kind,
+                             void* stream);
+
+/*
  * Which kernel kr_gemm_reduce_*_bf16 would run for a shape (contiguous operands), decided by the
  * same code that launches it; for benchmarks and logs that want to name the kernel they timed.
  * No counterpart in the reference (its tile sizes are keyword arguments of the wrappers,

@@ -112,6 +112,8 @@ _SIGNATURES = {
     "kr_cast_fp8_to_bf16": (c_int, [c_void_p, c_int64, c_void_p, c_void_p]),
     "kr_cast_f32_to_fp8": (c_int, [c_void_p, c_int64, c_void_p, c_void_p]),
     "kr_gemm_fp8": (c_int, [c_void_p, c_int64, c_void_p, c_int64, c_int64, c_int64, c_int64, c_void_p, c_int, c_void_p]),
+    "kr_all_gather_matmul_fp8": (c_int, [c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_int64, c_int64, c_int64, c_int64,
+                                         c_int, c_int, c_int, c_void_p, c_int64, c_void_p, c_void_p, c_int, c_void_p]),
     "kr_gemm_plan": (c_int, [c_int64, c_int64, c_int64, c_int, c_int, c_int64, c_int, c_int, c_int64, c_void_p]),
     "kr_probe_read": (c_int, [c_void_p, c_int64, c_void_p, c_void_p]),
     "kr_probe_copy": (c_int, [c_void_p, c_void_p, c_int64, c_void_p]),

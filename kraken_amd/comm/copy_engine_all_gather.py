@@ -49,7 +49,7 @@ def _copy_engine_all_gather_w_progress(
     are slower within one GPU.  ``progress`` must have been zeroed on the current
     stream beforehand.
     """
-    peers = PeerBuffers(inp)
+    peers = PeerBuffers(inp, dtypes=(torch.bfloat16, torch.float8_e4m3fn))
     W = peers.W
     assert 0 <= rank < W
     assert peers.cap % splits_per_rank == 0
@@ -58,7 +58,7 @@ def _copy_engine_all_gather_w_progress(
     out_shape = list(peers.slice(0).shape)
     out_shape[0] *= W
     assert list(output.shape) == out_shape, (list(output.shape), out_shape)
-    assert output.is_contiguous() and output.dtype == torch.bfloat16
+    assert output.is_contiguous() and output.dtype == peers.slice(0).dtype
     dev = _lib.require_device(*peers.tensors, output, progress)
     if backend_stream is None:
         backend_stream = _get_backend_stream(dev)

@@ -830,11 +830,12 @@ extern "C" int kr_gemm_producer_bf16(const void* A, int64_t lda_m, int64_t lda_k
                        0, ((int64_t)(rank + 1) % W) * (M / W), stream, &ps);
 }
 
-// Plain product of fp8 (e4m3fn) operands on the fp8 matrix-core instruction (all_gather_matmul.py:53,121,213: fp8 shards and
+// Product of fp8 (e4m3fn) operands on the fp8 matrix-core instruction (all_gather_matmul.py:53,121,213: fp8 shards and
 // weight, fp8 result).  The kernel is the 256x256 LDS-DMA kernel with its k-step on 16x16x128 blocks; it reads the operands
-// as matrices of two-byte units, hence the halved K and row strides below.
-extern "C" int kr_gemm_fp8(const void* A, int64_t lda, const void* Bt, int64_t ldb, int64_t M, int64_t N, int64_t K,
-                           void* out, int out_kind, void* stream) {
+// as matrices of two-byte units, hence the halved K and row strides below.  `gather`: rows of A that arrive while the
+// kernel runs (flags, local shard), as for the bf16 all-gather matmul.
+static int gemm_fp8(const void* A, int64_t lda, const void* Bt, int64_t ldb, int64_t M, int64_t N, int64_t K,
+                    void* out, int out_kind, void* stream, const GatherSpec* gather) {
     if (M < 0 || N < 0 || K < 0 || M > 0x7fffffffLL || N > 0x7fffffffLL || K > 0x7fffffffLL) return KR_ERR_BAD_DIM;
     if (out_kind < 0 || out_kind > 2) return KR_ERR_BAD_DIM;
     if (M % 256 != 0 || N % 256 != 0 || K % 128 != 0) return KR_ERR_BAD_DIM;
@@ -850,9 +851,21 @@ extern "C" int kr_gemm_fp8(const void* A, int64_t lda, const void* Bt, int64_t l
     g.lda = lda / 2;
     g.ldb = ldb / 2;
     g.M = (int)M; g.N = (int)N; g.K = (int)(K / 2);
-    if (!gemm_dtl_supported(g)) return KR_ERR_LAYOUT;
     g.comm_rows = 1;
     g.count_rows = 1;
+    int64_t pivot_row = 0;
+    if (gather != nullptr && gather->progress != nullptr) {
+        g.progress = gather->progress;
+        g.comm_rows = (int)gather->comm_rows;
+        g.a_local = (const uint16_t*)gather->a_local;
+        g.lda_local = gather->lda_local / 2;
+        g.local_row0 = (int)gather->local_row0;
+        g.local_rows = (int)gather->local_rows;
+        g.wait_ticks = (uint64_t)gather->wait_limit_us * 100u;   // 100 MHz constant clock
+        g.status = gather->status;
+    }
+    if (gather != nullptr) pivot_row = gather->local_row0;
+    if (!gemm_dtl_supported(g) || (g.a_local != nullptr && (int64_t)256 * g.lda_local * 2 >= 0x7fffffffLL)) return KR_ERR_LAYOUT;
     g.band_row0 = 0;
     g.band_rows = (int)M;
     g.out = out;
@@ -860,10 +873,39 @@ extern "C" int kr_gemm_fp8(const void* A, int64_t lda, const void* Bt, int64_t l
     g.out_fp8 = out_kind == 2;
     g.tiles_m = (int)(M / 256);
     g.tiles_n = (int)(N / 256);
+    g.pivot_tiles = (int)((pivot_row / 256) % g.tiles_m);
     g.group_n = env_switches().gemm_group > 0 ? env_switches().gemm_group : 4;
     g.k_splits = 1;
     g.mi16 = 1;
     return (int)launch_gemm_dtl8(g, (hipStream_t)stream);
+}
+
+extern "C" int kr_gemm_fp8(const void* A, int64_t lda, const void* Bt, int64_t ldb, int64_t M, int64_t N, int64_t K,
+                           void* out, int out_kind, void* stream) {
+    return gemm_fp8(A, lda, Bt, ldb, M, N, K, out, out_kind, stream, nullptr);
+}
+
+extern "C" int kr_all_gather_matmul_fp8(const void* A, int64_t lda, const void* A_local, int64_t lda_local, const void* Bt,
+                                        int64_t ldb, int64_t M, int64_t N, int64_t K, int W, int rank, int splits_per_rank,
+                                        const uint32_t* progress, int64_t wait_limit_us, int32_t* status, void* out,
+                                        int out_kind, void* stream) {
+    if (W < 1 || W > KR_MAX_WORLD) return KR_ERR_WORLD_SIZE;
+    if (rank < 0 || rank >= W || splits_per_rank < 1) return KR_ERR_STRIPE;
+    if (M < 0 || M % ((int64_t)W * splits_per_rank) != 0) return KR_ERR_BAND;
+    if (A_local != nullptr && (!aligned16(A_local) || lda_local % 16 != 0)) return KR_ERR_ALIGNMENT;
+    if (A_local != nullptr && lda_local < K) return KR_ERR_LAYOUT;
+    if ((reinterpret_cast<uintptr_t>(progress) & 3u) != 0 || (reinterpret_cast<uintptr_t>(status) & 3u) != 0)
+        return KR_ERR_ALIGNMENT;
+    GatherSpec gs{};
+    gs.a_local = A_local;
+    gs.lda_local = lda_local;
+    gs.local_rows = M / W;
+    gs.local_row0 = gs.local_rows * rank;
+    gs.progress = progress;
+    gs.comm_rows = M > 0 ? M / ((int64_t)W * splits_per_rank) : 1;
+    gs.wait_limit_us = wait_limit_us > 0 ? wait_limit_us : 5000000;   // 5 s
+    gs.status = status;
+    return gemm_fp8(A, lda, Bt, ldb, M, N, K, out, out_kind, stream, &gs);
 }
 
 extern "C" int kr_gemm_plan(int64_t M, int64_t N, int64_t K, int b_transposed, int n_peers, int64_t band_rows,

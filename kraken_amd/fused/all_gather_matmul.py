@@ -38,12 +38,14 @@ def _matmul_w_progress(a, a_local, b, progress, configs, status=None) -> torch.T
     return c
 
 
-def _all_gather_matmul_fp8(peers: PeerBuffers, b, a_out, progress, **kwargs):
+def _all_gather_matmul_fp8(a_shared, peers: PeerBuffers, b, a_out, progress, **kwargs):
     """The fp8 branch of ``all_gather_matmul`` (``all_gather_matmul.py:53,121,213``): fp8 product with fp32
     accumulation, rounded to fp8 once.  Shapes the fp8 kernel takes (M, N multiples of 256, K of 128) run on
-    the fp8 matrix-core instruction (``kr_gemm_fp8``); others are widened to bf16 (exact), multiplied by the
-    bf16 kernels with an fp32 result, and rounded by ``kr_cast_f32_to_fp8`` -- the same sums up to fp32
-    summation order.  ``fp8_kernel=False`` forces the widening path."""
+    the fp8 matrix-core instruction (``kr_gemm_fp8``, or ``kr_all_gather_matmul_fp8`` for ``gather=True``: the
+    shards are copied chunk by chunk on a side stream while the tiles wait for their chunk's flag, as in the
+    bf16 form); others are widened to bf16 (exact), multiplied by the bf16 kernels with an fp32 result, and
+    rounded by ``kr_cast_f32_to_fp8`` -- the same sums up to fp32 summation order -- after the gather has
+    finished.  ``fp8_kernel=False`` forces the widening path."""
     fp8 = torch.float8_e4m3fn
     W = peers.W
     m, K = peers.slice(0).shape
@@ -52,24 +54,58 @@ def _all_gather_matmul_fp8(peers: PeerBuffers, b, a_out, progress, **kwargs):
     if not b.T.is_contiguous():
         raise ValueError("b.T must be contiguous")
     stacked = peers.stacked is not None and peers.stacked.is_contiguous()
-    if kwargs.get("gather", not stacked) or not stacked:
-        raise NotImplementedError("fp8 shards: only the gathered form (one contiguous [W, m, K] tensor, gather=False)")
+    gather = kwargs.get("gather", not stacked)
     M, N = W * m, b.shape[1]
     assert K % 16 == 0 and N % 16 == 0 and (M * N) % 16 == 0, "fp8 operands: sizes must be multiples of 16"
     rank = kwargs.get("rank", 0)
     assert 0 <= rank < W
-    dev = _lib.require_device(peers.stacked, b, a_out, progress)
+    splits = kwargs.get("splits_per_rank", 1)
+    dev = _lib.require_device(*peers.tensors, b, a_out, progress)
     lib = _lib.load()
     stream = _lib.current_stream(dev)
-    a_full = peers.stacked.reshape(M, K)
-    if a_out is not None:
-        assert a_out.shape == a_full.shape and a_out.dtype == fp8
-        a_out.copy_(a_full)
+    native = kwargs.get("fp8_kernel", True) and M % 256 == 0 and N % 256 == 0 and K % 128 == 0
+    if gather:
+        assert m % splits == 0, "splits_per_rank must divide the rows of a shard"
+        _waits.check()      # an earlier call's failed wait is reported before anything of this call is enqueued
+        if a_out is None:
+            a_out = torch.empty((M, K), dtype=fp8, device=dev)
+        else:
+            assert tuple(a_out.shape) == (M, K) and a_out.dtype == fp8 and a_out.is_contiguous()
+        if progress is None:
+            progress = torch.zeros(W * splits, dtype=torch.int32, device=dev)
+        else:
+            progress.fill_(0)
+        backend_stream = _copy_engine_all_gather_w_progress(a_out, a_shared, progress, splits, rank=rank,
+                                                            copy_engine=kwargs.get("copy_engine", False))
+        if native:
+            status = kwargs.get("status")
+            own_status = status is None
+            if own_status:
+                status = _waits.new_status(dev)
+            a_local = peers.slice(rank)
+            assert a_local.stride(1) == 1
+            c = torch.empty((M, N), dtype=fp8, device=dev)
+            rc = lib.kr_all_gather_matmul_fp8(
+                a_out.data_ptr(), K, a_local.data_ptr(), a_local.stride(0), b.T.data_ptr(), K, M, N, K, W, rank, splits,
+                progress.data_ptr(), int(kwargs.get("wait_limit_us", 0)), _lib.ptr(status), c.data_ptr(), 2, stream)
+            _lib.check(rc, "all_gather_matmul(fp8)")
+            torch.cuda.current_stream(dev).wait_stream(backend_stream)
+            if own_status:
+                _waits.watch(status, "all_gather_matmul")
+            return a_out, c
+        torch.cuda.current_stream(dev).wait_stream(backend_stream)   # no overlap on the widening path
+        a_full = a_out
     else:
-        a_out = a_full
-    if progress is not None:
-        progress.fill_(1)
-    if kwargs.get("fp8_kernel", True) and M % 256 == 0 and N % 256 == 0 and K % 128 == 0:
+        assert stacked, "gather=False needs the shards as one contiguous [W, m, K] tensor"
+        a_full = peers.stacked.reshape(M, K)
+        if a_out is not None:
+            assert a_out.shape == a_full.shape and a_out.dtype == fp8
+            a_out.copy_(a_full)
+        else:
+            a_out = a_full
+        if progress is not None:
+            progress.fill_(1)
+    if native:
         c = torch.empty((M, N), dtype=fp8, device=dev)
         _lib.check(lib.kr_gemm_fp8(a_full.data_ptr(), K, b.T.data_ptr(), K, M, N, K, c.data_ptr(), 2, stream),
                    "all_gather_matmul(fp8)")
@@ -125,16 +161,17 @@ def all_gather_matmul(
 
     fp8 operands (``torch.float8_e4m3fn`` for the shards and ``b``) give an fp8 ``c``
     like in the reference (``:53,121,213``): fp32 accumulate, one rounding to fp8
-    (nearest even, magnitudes of 448 and more saturate to 448).  Here the operands
-    are widened to bf16 by one conversion pass each (exact: every e4m3 value is a
-    bf16 value), the bf16 kernels run with an fp32 result, and a third pass rounds
-    that to fp8; ``a_gathered`` stays fp8.  Only for ``gather=False`` and sizes that
-    are multiples of 16.
+    (nearest even, magnitudes of 448 and more saturate to 448), in both modes.
+    With M and N multiples of 256 and K of 128 the product runs on the fp8
+    matrix-core instruction; other sizes (multiples of 16) are widened to bf16 by one
+    conversion pass per operand (exact: every e4m3 value is a bf16 value), multiplied
+    by the bf16 kernels with an fp32 result and rounded to fp8 by a third pass, after
+    the gather has finished.  ``a_gathered`` stays fp8.
     """
     fp8 = torch.float8_e4m3fn
     peers = PeerBuffers(a_shared, dtypes=(torch.bfloat16, fp8))
     if peers.slice(0).dtype == fp8:
-        return _all_gather_matmul_fp8(peers, b, a_out, progress, **kwargs)
+        return _all_gather_matmul_fp8(a_shared, peers, b, a_out, progress, **kwargs)
     W = peers.W
     shard = peers.slice(0)
     assert shard.dim() == 2, "expected shards of shape [m, K]"

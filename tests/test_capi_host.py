@@ -371,6 +371,19 @@ def test_gemm_fp8_argument_errors(lib):
     assert call(ldb=520) == _lib.KR_ERR_ALIGNMENT        # row stride not a multiple of 16 bytes
     assert call(Bt=FAKE + 8) == _lib.KR_ERR_ALIGNMENT
     assert call(M=0, A=None, Bt=None, out=None) == 0     # nothing to do, nothing launched
+    g = lib.kr_all_gather_matmul_fp8
+    base = dict(A=FAKE, lda=512, A_local=FAKE, lda_local=512, Bt=FAKE, ldb=512, M=2048, N=256, K=512, W=8, rank=3, splits=1,
+                progress=FAKE, limit=0, status=None, out=FAKE, kind=2, stream=None)
+    def gcall(**kw):
+        args = dict(base); args.update(kw)
+        return g(*args.values())
+    assert gcall(W=0) == _lib.KR_ERR_WORLD_SIZE
+    assert gcall(rank=8) == _lib.KR_ERR_STRIPE
+    assert gcall(splits=3) == _lib.KR_ERR_BAND           # 2048 rows in 24 chunks
+    assert gcall(lda_local=520) == _lib.KR_ERR_ALIGNMENT
+    assert gcall(lda_local=256) == _lib.KR_ERR_LAYOUT
+    assert gcall(progress=FAKE + 2) == _lib.KR_ERR_ALIGNMENT
+    assert gcall(M=1024, N=384) == _lib.KR_ERR_BAD_DIM   # the product's own shape rule
 
 
 def test_probe_argument_errors(lib):

@@ -151,8 +151,6 @@ def test_all_gather_matmul_fp8(dev):
     assert (got == ref).float().mean() > 0.99
     step = torch.maximum(ref.abs(), torch.tensor(2.0 ** -6)) * 2.0 ** -3          # spacing of e4m3 at that magnitude
     assert ((got - ref).abs() <= step).all()
-    with pytest.raises(NotImplementedError):
-        fused.all_gather_matmul(a.to(dev), bT.to(dev).T, gather=True)
 
 
 @pytest.mark.parametrize("K", [128, 256, 384, 1024])
@@ -217,6 +215,40 @@ def test_fp8_kernel_random_operands_and_nan(dev):
     assert lib.kr_gemm_fp8(a_nan.to(dev).data_ptr(), K, bT.to(dev).data_ptr(), K, M, N, K, c.data_ptr(), 2, stream) == 0
     nan = torch.isnan(c.cpu().float())
     assert nan[300].all() and not nan[:300].any() and not nan[301:].any()
+
+
+@pytest.mark.parametrize("splits", [1, 2])
+@pytest.mark.parametrize("as_list", [False, True])
+def test_all_gather_matmul_fp8_overlapped(dev, splits, as_list):
+    """gather=True with fp8 shards (the reference's overlap, all_gather_matmul.py:308-323, on its fp8 branch):
+    the chunks are copied on the side stream and flagged while the fp8 kernel's tiles wait for them; the
+    gathered matrix is the shards bit for bit, every flag ends at 1, and the product has the bits of the
+    gather=False call (same kernel, same sums).  Also a shape the fp8 kernel does not take (the widening
+    path behind the finished gather)."""
+    from kraken_amd import _waits
+    fp8 = torch.float8_e4m3fn
+    W, m, K, N = 8, 256, 1024, 768
+    g = torch.Generator().manual_seed(51)
+    a = torch.randn(W, m, K, generator=g).to(fp8)
+    bT = (torch.randn(N, K, generator=g) * 0.05).to(fp8)
+    ad, bd = a.to(dev), bT.to(dev)
+    _, want = fused.all_gather_matmul(ad, bd.T, rank=5)
+    shards = [ad[r].clone() for r in range(W)] if as_list else ad
+    progress = torch.zeros(W * splits, dtype=torch.int32, device=dev)
+    a_out, c = fused.all_gather_matmul(shards, bd.T, None, progress, rank=5, splits_per_rank=splits, gather=True)
+    torch.cuda.synchronize()
+    _waits.check(block=True)
+    assert a_out.dtype == fp8 and torch.equal(a_out.cpu().view(torch.uint8), a.reshape(W * m, K).view(torch.uint8))
+    assert (progress.cpu() == 1).all()
+    assert torch.equal(c.cpu().view(torch.uint8), want.cpu().view(torch.uint8))
+    _, ref = orc.all_gather_matmul_fp8(a, bT.T)
+    assert (c.cpu().float() == ref.float()).float().mean() > 0.99
+    # 8 x 48 rows: not a multiple of 256
+    a2, b2 = a[:, :48].contiguous(), bT[:400]
+    a_out, c = fused.all_gather_matmul(a2.to(dev), b2.to(dev).T, rank=1, gather=True)
+    _, ref = orc.all_gather_matmul_fp8(a2, b2.T)
+    assert torch.equal(a_out.cpu().view(torch.uint8), a2.reshape(-1, K).view(torch.uint8))
+    assert (c.cpu().float() == ref.float()).float().mean() > 0.99
 
 
 def test_split_fp32_is_one_pass_and_bit_exact(dev):
