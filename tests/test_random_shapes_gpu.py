@@ -185,3 +185,31 @@ def test_large_tile_kernel_random_shapes_and_switches(dev, monkeypatch, seed):
                                    rtol=1e-3, atol=1e-3)
         torch.testing.assert_close(fused.gemm_one_shot_all_reduce_fused(ad, bd, peers=pd, bias=bsd, out_dtype=BF16).cpu(),
                                    want.to(BF16), **TOL)
+
+
+@pytest.mark.parametrize("seed", range(10))
+def test_fp8_kernel_random_shapes(dev, seed):
+    """kr_gemm_fp8 on random whole-tile shapes, row strides and result types: small integers and halves, so every
+    fp32 sum is exact and the result must equal the product bit for bit (fp8 results: the saturating conversion
+    of the exact product); tile counts on either side of a round of 256 compute units, odd and even k-step counts."""
+    from kraken_amd import _lib
+    fp8 = torch.float8_e4m3fn
+    rnd = random.Random(5000 + seed)
+    M, N, K = 256 * rnd.randint(1, 12), 256 * rnd.randint(1, 12), 128 * rnd.randint(1, 9)
+    lda, ldb = K + 16 * rnd.randint(0, 3), K + 16 * rnd.randint(0, 3)
+    g = torch.Generator().manual_seed(seed)
+    a = torch.zeros(M, lda).to(fp8)
+    b = torch.zeros(N, ldb).to(fp8)
+    a[:, :K] = torch.randint(-2, 3, (M, K), generator=g).float().to(fp8)
+    b[:, :K] = (torch.randint(-3, 4, (N, K), generator=g).float() * 0.5).to(fp8)
+    a[:, K:], b[:, K:] = 3.0, 3.0                 # what lies between the rows must not be read
+    exact = a[:, :K].float() @ b[:, :K].float().T
+    lib = _lib.load()
+    stream = torch.cuda.current_stream(dev).cuda_stream
+    ad, bd = a.to(dev), b.to(dev)
+    kind = rnd.choice([0, 1, 2])
+    dtype = (BF16, torch.float32, fp8)[kind]
+    out = torch.empty(M, N, dtype=dtype, device=dev)
+    assert lib.kr_gemm_fp8(ad.data_ptr(), lda, bd.data_ptr(), ldb, M, N, K, out.data_ptr(), kind, stream) == 0, (M, N, K)
+    want = exact.clamp(-448.0, 448.0).to(fp8) if kind == 2 else exact.to(dtype)
+    assert torch.equal(out.cpu().float(), want.float()), (M, N, K, lda, ldb, kind)
