@@ -735,8 +735,8 @@ def time_gpu_eager(step, steps, warmup, settle_ms=SETTLE_MS):
 
     An event between two launches costs about 2 us of GPU time on this machine (the launches no
     longer run back to back), which would be charged to the kernel: an interval therefore covers
-    as many launches as it takes to last MIN_INTERVAL_MS -- one for the GEMMs, five for a 50 us
-    kernel -- so that the markers stay below one percent of what they bracket.
+    as many launches as it takes to last MIN_INTERVAL_MS, and at least two -- two for the GEMMs,
+    five for a 50 us kernel -- so that the markers stay below one percent of what they bracket.
     """
     import torch
 
@@ -750,7 +750,7 @@ def time_gpu_eager(step, steps, warmup, settle_ms=SETTLE_MS):
     b.record()
     torch.cuda.synchronize()
     est_ms = a.elapsed_time(b) / 10
-    stride = max(1, min(steps, int(-(-MIN_INTERVAL_MS // est_ms))))
+    stride = max(2 if steps >= 8 else 1, min(steps, int(-(-MIN_INTERVAL_MS // est_ms))))
     marks = list(range(0, steps, stride)) + [steps]          # an event in front of these steps, and one at the end
     evs = [torch.cuda.Event(enable_timing=True) for _ in marks]
     torch.cuda.synchronize()
