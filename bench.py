@@ -751,7 +751,8 @@ def time_gpu_eager(step, steps, warmup, settle_ms=SETTLE_MS):
     torch.cuda.synchronize()
     est_ms = a.elapsed_time(b) / 10
     stride = max(2 if steps >= 8 else 1, min(steps, int(-(-MIN_INTERVAL_MS // est_ms))))
-    marks = list(range(0, steps, stride)) + [steps]          # an event in front of these steps, and one at the end
+    n_int = -(-steps // stride)                               # intervals of equal length (to within one launch)
+    marks = [j * steps // n_int for j in range(n_int)] + [steps]   # an event in front of these steps, and one at the end
     evs = [torch.cuda.Event(enable_timing=True) for _ in marks]
     torch.cuda.synchronize()
     t0 = time.perf_counter()
@@ -766,7 +767,7 @@ def time_gpu_eager(step, steps, warmup, settle_ms=SETTLE_MS):
     t1 = time.perf_counter()
     per = [evs[j].elapsed_time(evs[j + 1]) / (marks[j + 1] - marks[j]) for j in range(len(marks) - 1)]
     st = _stats(per)
-    st["launches_per_interval"] = stride
+    st["launches_per_interval"] = steps // n_int
     return (t1 - t0) * 1e3 / steps, st, steps
 
 
