@@ -578,8 +578,10 @@ static GemmPlan plan_gemm(int64_t M, int64_t N, int64_t K, bool b_nt, int n_peer
     // 256 compute units (8192 x 3584: 448 tiles = 2 rounds of 256 columns against 512 tiles = 2
     // rounds of 224: measured 340 -> 320 us at K = 8192); a 224-column tile costs about 3 % more
     // per flop (A is read from LDS and L2 for fewer columns).  KRAKEN_AMD_GEMM_N224=0|1 overrides.
+    // (An A that arrives while the kernel runs is fine: the tile waits for its rows' flags before its
+    // first load, whatever its width.)
     p.n224 = 0;
-    if (dtl && p.mi16 && b_nt && plain && plain_bf16_all_rows && !has_gather && M % 256 == 0 && N % 224 == 0) {
+    if (dtl && p.mi16 && b_nt && plain && plain_bf16_all_rows && M % 256 == 0 && N % 224 == 0) {
         const int64_t t8 = tiles_m * tiles_n, t7 = (M / 256) * (N / 224);
         const double cost8 = (double)((t8 + 255) / 256) * 256.0, cost7 = (double)((t7 + 255) / 256) * 224.0 * 1.03;
         bool use = cost7 < cost8;

@@ -80,6 +80,9 @@ def test_all_gather_matmul_224_column_tiles(dev, monkeypatch):
     _, want = orc.all_gather_matmul(stack, bT.T)
     torch.testing.assert_close(c.cpu().float(), want.float(), **TOL)
     assert torch.equal(a_out.cpu(), stack.reshape(W * m, K))
+    # the overlapped form takes the same tiles (a tile waits for its rows' flags before its first load)
+    a_g, c_g = fused.all_gather_matmul(stack.to(dev), bT.to(dev).T, rank=5, gather=True, splits_per_rank=2)
+    assert torch.equal(c, c_g) and torch.equal(a_g.cpu(), stack.reshape(W * m, K))
     monkeypatch.setenv("KRAKEN_AMD_GEMM_N224", "0")
     assert _lib.gemm_plan(W * m, N, K, True)["kernel"] == "gemm_dtl16_kernel"
     _, c256 = fused.all_gather_matmul(stack.to(dev), bT.to(dev).T, rank=5)
